@@ -1,0 +1,63 @@
+// Python bindings for the sequence-mixer kernels (dynamo_amd._hip_seq):
+// recurrent matrix-state mixers, biased paged attention and their row-wise
+// companions. Built apart from dynamo_amd._hip so that a model which only
+// needs these compiles in seconds.
+#include <torch/extension.h>
+#include <pybind11/pybind11.h>
+
+using torch::Tensor;
+using OptTensor = c10::optional<torch::Tensor>;
+
+void embed_scale_pos(Tensor out, Tensor ids, Tensor positions, Tensor embed,
+                     OptTensor pos, double scale);
+void add_scalar_rmsnorm(Tensor out, Tensor res, OptTensor delta, Tensor g,
+                        double eps);
+void causal_conv_silu(Tensor out, Tensor x, Tensor w, Tensor conv_state,
+                      Tensor tok_seq, Tensor seq_start, Tensor seq_len,
+                      Tensor seq_slot, Tensor seq_pos0);
+void token_shift_mix(Tensor out, Tensor h, Tensor mu, Tensor prev_state,
+                     Tensor tok_seq, Tensor seq_start, Tensor seq_len,
+                     Tensor seq_slot, Tensor seq_pos0);
+void head_norm_gate(Tensor out, Tensor o, Tensor w, int64_t w_stride,
+                    OptTensor gate, int64_t gate_act, double eps);
+void clamped_glu(Tensor out, Tensor gate_up, double limit, double alpha);
+void dual_rmsnorm_mean(Tensor out, Tensor a, Tensor b, Tensor wa, Tensor wb,
+                       double eps);
+void softcap_(Tensor x, double cap);
+void gated_delta_rule(Tensor out, Tensor qkv, Tensor proj, int64_t off_b,
+                      int64_t off_a, Tensor A_log, Tensor dt_bias, Tensor state,
+                      Tensor seq_start, Tensor seq_len, Tensor seq_slot,
+                      Tensor seq_pos0, int64_t G, double qscale,
+                      double unit_eps);
+void rwkv_time_mix(Tensor out, Tensor r, Tensor k, Tensor v, Tensor wraw,
+                   Tensor w0, Tensor u, Tensor state, Tensor seq_start,
+                   Tensor seq_len, Tensor seq_slot, Tensor seq_pos0);
+void mlstm_memory(Tensor out, Tensor proj, int64_t off_q, int64_t off_k,
+                  int64_t off_v, int64_t off_i, int64_t off_f, Tensor i_bias,
+                  Tensor f_bias, Tensor state_S, Tensor state_n, Tensor state_m,
+                  Tensor seq_start, Tensor seq_len, Tensor seq_slot,
+                  Tensor seq_pos0, double qscale, double cap, double den_eps);
+void kv_append_norm(Tensor kcache, Tensor vcache, Tensor proj, int64_t off_k,
+                    int64_t off_v, Tensor slot_mapping, bool vnorm, double eps);
+void biased_attention(Tensor out, Tensor proj, int64_t off_q, Tensor kcache,
+                      Tensor vcache, Tensor page_table, Tensor tok_seq,
+                      Tensor positions, Tensor seq_len, OptTensor r1,
+                      OptTensor r2, double scale, double temp_coef,
+                      int64_t temp_every);
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.doc() = "dynamo_amd sequence-mixer kernels (gfx950)";
+  m.def("embed_scale_pos", &embed_scale_pos);
+  m.def("add_scalar_rmsnorm", &add_scalar_rmsnorm);
+  m.def("causal_conv_silu", &causal_conv_silu);
+  m.def("token_shift_mix", &token_shift_mix);
+  m.def("head_norm_gate", &head_norm_gate);
+  m.def("clamped_glu", &clamped_glu);
+  m.def("dual_rmsnorm_mean", &dual_rmsnorm_mean);
+  m.def("softcap_", &softcap_);
+  m.def("gated_delta_rule", &gated_delta_rule);
+  m.def("rwkv_time_mix", &rwkv_time_mix);
+  m.def("mlstm_memory", &mlstm_memory);
+  m.def("kv_append_norm", &kv_append_norm);
+  m.def("biased_attention", &biased_attention);
+}

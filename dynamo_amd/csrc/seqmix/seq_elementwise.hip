@@ -1,0 +1,411 @@
+// Row-wise kernels of the sequence-mixer models: embedding, scalar-gain RMS
+// norm fused with the fp32 residual add, short causal convolution, token
+// shift, per-head output norm with gate, clamped GLU, two-branch merge and
+// the logit soft cap. All of them are bandwidth bound; one workgroup per
+// token row, fp32 arithmetic, activations in T.
+#include "seq_common.h"
+
+namespace {
+
+// x[t] = embed[id[t]] * scale + pos[position[t]]  (fp32 residual stream)
+template <typename T>
+__global__ void embed_scale_pos_kernel(float* __restrict__ out,
+                                       const int* __restrict__ ids,
+                                       const int* __restrict__ positions,
+                                       const T* __restrict__ embed,
+                                       const T* __restrict__ pos, float scale,
+                                       int W, int has_pos) {
+  const int t = blockIdx.x;
+  const T* e = embed + (int64_t)ids[t] * W;
+  const T* p = pos + (int64_t)positions[t] * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float v = to_f(e[i]) * scale;
+    if (has_pos) v += to_f(p[i]);
+    out[(int64_t)t * W + i] = v;
+  }
+}
+
+// res += delta (when given); out = res / sqrt(mean(res^2) + eps) * g[0]
+template <typename T, bool ADD>
+__global__ void add_scalar_rmsnorm_kernel(T* __restrict__ out,
+                                          float* __restrict__ res,
+                                          const T* __restrict__ delta,
+                                          const float* __restrict__ g,
+                                          float eps, int W) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  float* r = res + (int64_t)t * W;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float v = r[i];
+    if (ADD) {
+      v += to_f(delta[(int64_t)t * W + i]);
+      r[i] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = g[0] / sqrtf(ss / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x)
+    out[(int64_t)t * W + i] = from_f<T>(r[i] * inv);
+}
+
+// y[t, c] = silu(sum_j w[c, j] * x[t - (taps-1) + j, c]); rows before the
+// start of this step's portion come from the slot's saved inputs (the last
+// taps-1 raw inputs of the sequence), or are zero at position 0.
+template <typename T>
+__global__ void causal_conv_silu_kernel(
+    float* __restrict__ out, const T* __restrict__ x, int x_stride,
+    const float* __restrict__ w, const float* __restrict__ conv_state,
+    const int* __restrict__ tok_seq, const int* __restrict__ seq_start,
+    const int* __restrict__ seq_slot, const int* __restrict__ seq_pos0,
+    int C, int taps) {
+  const int t = blockIdx.x;
+  const int s = tok_seq[t];
+  const int start = seq_start[s], pos0 = seq_pos0[s];
+  const float* st = conv_state + (int64_t)seq_slot[s] * (taps - 1) * C;
+  const int rel = t - start;  // rows of this portion before t
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float acc = 0.f;
+    for (int j = 0; j < taps; j++) {
+      const int back = taps - 1 - j;  // how many tokens before t
+      float xv;
+      if (back <= rel) {
+        xv = to_f(x[(int64_t)(t - back) * x_stride + c]);
+      } else {
+        // state row i holds the input (taps-1-i) tokens before the portion
+        const int before = back - rel;  // 1..taps-1 tokens before the start
+        xv = (pos0 - before >= 0) ? st[(int64_t)(taps - 1 - before) * C + c]
+                                  : 0.f;
+      }
+      acc += w[c * taps + j] * xv;
+    }
+    out[(int64_t)t * C + c] = silu_f(acc);
+  }
+}
+
+// After a step: the slot keeps the last taps-1 raw inputs of each sequence.
+template <typename T>
+__global__ void conv_state_update_kernel(
+    float* __restrict__ conv_state, const T* __restrict__ x, int x_stride,
+    const int* __restrict__ seq_start, const int* __restrict__ seq_len,
+    const int* __restrict__ seq_slot, const int* __restrict__ seq_pos0, int C,
+    int taps) {
+  const int s = blockIdx.x;
+  const int len = seq_len[s];
+  if (len == 0) return;
+  const int start = seq_start[s], pos0 = seq_pos0[s];
+  float* st = conv_state + (int64_t)seq_slot[s] * (taps - 1) * C;
+  const int K = taps - 1;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    // new row i holds the input (K - i) tokens before the NEXT portion;
+    // rows are filled in rising order, each reading only old rows above it
+    for (int i = 0; i < K; i++) {
+      const int back = K - i;  // tokens before the end of this portion
+      float v;
+      if (back <= len) {
+        v = to_f(x[(int64_t)(start + len - back) * x_stride + c]);
+      } else {
+        const int before = back - len;  // tokens before this portion's start
+        v = (pos0 - before >= 0) ? st[(int64_t)(K - before) * C + c] : 0.f;
+      }
+      st[(int64_t)i * C + c] = v;
+    }
+  }
+}
+
+// Token shift: mix_s[t] = h[t] + (h[t-1] - h[t]) * mu_s, S mixes at once.
+// The row before a portion comes from the slot (zero at position 0).
+template <typename T>
+__global__ void token_shift_mix_kernel(
+    T* __restrict__ out,  // [S, Ttot, W]
+    const T* __restrict__ h, const float* __restrict__ mu,  // [S, W]
+    const float* __restrict__ prev_state,                   // [slots, W]
+    const int* __restrict__ tok_seq, const int* __restrict__ seq_start,
+    const int* __restrict__ seq_slot, const int* __restrict__ seq_pos0,
+    int Ttot, int W, int S) {
+  const int t = blockIdx.x;
+  const int s = tok_seq[t];
+  const bool first = (t == seq_start[s]);
+  const bool zero = first && seq_pos0[s] == 0;
+  const float* ps = prev_state + (int64_t)seq_slot[s] * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float cur = to_f(h[(int64_t)t * W + i]);
+    const float prev =
+        zero ? 0.f : (first ? ps[i] : to_f(h[(int64_t)(t - 1) * W + i]));
+    for (int k = 0; k < S; k++)
+      out[((int64_t)k * Ttot + t) * W + i] =
+          from_f<T>(cur + (prev - cur) * mu[k * W + i]);
+  }
+}
+
+template <typename T>
+__global__ void shift_state_update_kernel(
+    float* __restrict__ prev_state, const T* __restrict__ h,
+    const int* __restrict__ seq_start, const int* __restrict__ seq_len,
+    const int* __restrict__ seq_slot, int W) {
+  const int s = blockIdx.x;
+  const int len = seq_len[s];
+  if (len == 0) return;
+  const T* last = h + (int64_t)(seq_start[s] + len - 1) * W;
+  float* ps = prev_state + (int64_t)seq_slot[s] * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) ps[i] = to_f(last[i]);
+}
+
+// y[t, h, :] = o[t, h, :] / rms(o[t, h, :]) * w[h * w_stride + :] * act(gate)
+// gate_act: 0 none, 1 silu, 2 sigmoid. One wave per (token, head).
+template <typename T>
+__global__ void head_norm_gate_kernel(T* __restrict__ out,
+                                      const float* __restrict__ o,
+                                      const float* __restrict__ w, int w_stride,
+                                      const T* __restrict__ gate,
+                                      int gate_stride, int gate_act, float eps,
+                                      int H, int dv) {
+  const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+  const float* src = o + ((int64_t)t * H + hh) * dv;
+  float ss = 0.f;
+  for (int i = lane; i < dv; i += 64) ss += src[i] * src[i];
+  ss = wave_sum(ss);
+  const float inv = 1.f / sqrtf(ss / (float)dv + eps);
+  for (int i = lane; i < dv; i += 64) {
+    float v = src[i] * inv * w[hh * w_stride + i];
+    if (gate_act) {
+      const float gr = to_f(gate[(int64_t)t * gate_stride + hh * dv + i]);
+      v *= (gate_act == 1) ? silu_f(gr) : sigmoid_f(gr);
+    }
+    out[((int64_t)t * H + hh) * dv + i] = from_f<T>(v);
+  }
+}
+
+// g = min(gate, L); u = clamp(up, -L, L); y = g * sigmoid(alpha g) * (u + 1)
+template <typename T>
+__global__ void clamped_glu_kernel(T* __restrict__ out,
+                                   const T* __restrict__ gate_up, int F,
+                                   float limit, float alpha, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int64_t t = i / F;
+  const int c = (int)(i - t * F);
+  const float g = fminf(to_f(gate_up[t * 2 * F + c]), limit);
+  const float u = fminf(fmaxf(to_f(gate_up[t * 2 * F + F + c]), -limit), limit);
+  out[i] = from_f<T>(g * sigmoid_f(alpha * g) * (u + 1.f));
+}
+
+// out = 0.5 * (a / rms(a) * wa + b / rms(b) * wb)
+template <typename T>
+__global__ void dual_rmsnorm_mean_kernel(T* __restrict__ out,
+                                         const T* __restrict__ a,
+                                         const T* __restrict__ b,
+                                         const float* __restrict__ wa,
+                                         const float* __restrict__ wb,
+                                         float eps, int W) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  float sa = 0.f, sb = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float x = to_f(a[(int64_t)t * W + i]);
+    const float y = to_f(b[(int64_t)t * W + i]);
+    sa += x * x;
+    sb += y * y;
+  }
+  sa = block_sum(sa, scratch);
+  sb = block_sum(sb, scratch);
+  const float ia = 1.f / sqrtf(sa / (float)W + eps);
+  const float ib = 1.f / sqrtf(sb / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float x = to_f(a[(int64_t)t * W + i]) * ia * wa[i];
+    const float y = to_f(b[(int64_t)t * W + i]) * ib * wb[i];
+    out[(int64_t)t * W + i] = from_f<T>(0.5f * (x + y));
+  }
+}
+
+__global__ void softcap_kernel(float* __restrict__ x, float cap, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = cap * tanhf(x[i] / cap);
+}
+
+inline int row_block(int W) {
+  int b = 64;
+  while (b < W && b < 1024) b <<= 1;
+  return b;
+}
+
+}  // namespace
+
+void embed_scale_pos(torch::Tensor out, torch::Tensor ids,
+                     torch::Tensor positions, torch::Tensor embed,
+                     c10::optional<torch::Tensor> pos, double scale) {
+  const int T_ = ids.size(0), W = embed.size(1);
+  SEQ_CHECK(out.scalar_type() == torch::kFloat && out.is_contiguous() &&
+                out.size(0) == T_ && out.size(1) == W, "embed out");
+  SEQ_CHECK(ids.scalar_type() == torch::kInt &&
+                positions.scalar_type() == torch::kInt &&
+                positions.size(0) == T_, "embed ids/positions int32");
+  SEQ_CHECK(embed.is_contiguous(), "embed table");
+  if (pos) SEQ_CHECK(pos->is_contiguous() && pos->size(1) == W &&
+                         pos->scalar_type() == embed.scalar_type(), "pos table");
+  if (T_ == 0) return;
+  DISPATCH_ACT(embed, hipLaunchKernelGGL(
+      embed_scale_pos_kernel<T>, dim3(T_), dim3(row_block(W)), 0, cur_stream(),
+      ptr<float>(out), cptr<int>(ids), cptr<int>(positions), cptr<T>(embed),
+      pos ? cptr<T>(*pos) : cptr<T>(embed), (float)scale, W, pos ? 1 : 0););
+}
+
+void add_scalar_rmsnorm(torch::Tensor out, torch::Tensor res,
+                        c10::optional<torch::Tensor> delta, torch::Tensor g,
+                        double eps) {
+  const int T_ = res.size(0), W = res.size(1);
+  SEQ_CHECK(res.scalar_type() == torch::kFloat && res.is_contiguous(), "res");
+  SEQ_CHECK(out.is_contiguous() && out.size(0) == T_ && out.size(1) == W, "out");
+  SEQ_CHECK(g.scalar_type() == torch::kFloat && g.numel() == 1, "gain");
+  if (delta)
+    SEQ_CHECK(delta->is_contiguous() && delta->size(0) == T_ &&
+                  delta->size(1) == W &&
+                  delta->scalar_type() == out.scalar_type(), "delta");
+  if (T_ == 0) return;
+  DISPATCH_ACT(out, {
+    if (delta)
+      hipLaunchKernelGGL((add_scalar_rmsnorm_kernel<T, true>), dim3(T_),
+                         dim3(row_block(W)), 0, cur_stream(), ptr<T>(out),
+                         ptr<float>(res), cptr<T>(*delta), cptr<float>(g),
+                         (float)eps, W);
+    else
+      hipLaunchKernelGGL((add_scalar_rmsnorm_kernel<T, false>), dim3(T_),
+                         dim3(row_block(W)), 0, cur_stream(), ptr<T>(out),
+                         ptr<float>(res), (const T*)nullptr, cptr<float>(g),
+                         (float)eps, W);
+  });
+}
+
+static void check_seq(const torch::Tensor& a, int64_t n, const char* what) {
+  TORCH_CHECK(a.scalar_type() == torch::kInt && a.is_contiguous() &&
+                  a.numel() >= n, "seqmix: ", what, " must be int32 [>=", n, "]");
+}
+
+void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                      torch::Tensor conv_state, torch::Tensor tok_seq,
+                      torch::Tensor seq_start, torch::Tensor seq_len,
+                      torch::Tensor seq_slot, torch::Tensor seq_pos0) {
+  // x: [T, >=C] rows of stride x.stride(0); the first C columns convolve
+  const int T_ = x.size(0), C = w.size(0), taps = w.size(1);
+  const int B = seq_start.size(0);
+  SEQ_CHECK(x.stride(1) == 1 && x.size(1) >= C, "conv input");
+  SEQ_CHECK(out.scalar_type() == torch::kFloat && out.is_contiguous() &&
+                out.size(0) == T_ && out.size(1) == C, "conv out");
+  SEQ_CHECK(w.scalar_type() == torch::kFloat && w.is_contiguous(), "conv w");
+  SEQ_CHECK(conv_state.scalar_type() == torch::kFloat &&
+                conv_state.is_contiguous() && conv_state.size(1) == taps - 1 &&
+                conv_state.size(2) == C, "conv state");
+  check_seq(tok_seq, T_, "tok_seq");
+  check_seq(seq_len, B, "seq_len");
+  check_seq(seq_slot, B, "seq_slot");
+  check_seq(seq_pos0, B, "seq_pos0");
+  if (T_ == 0) return;
+  DISPATCH_ACT(x, {
+    hipLaunchKernelGGL(causal_conv_silu_kernel<T>, dim3(T_), dim3(row_block(C)),
+                       0, cur_stream(), ptr<float>(out), cptr<T>(x),
+                       (int)x.stride(0), cptr<float>(w),
+                       cptr<float>(conv_state), cptr<int>(tok_seq),
+                       cptr<int>(seq_start), cptr<int>(seq_slot),
+                       cptr<int>(seq_pos0), C, taps);
+    if (taps > 1)
+      hipLaunchKernelGGL(conv_state_update_kernel<T>, dim3(B),
+                         dim3(row_block(C)), 0, cur_stream(),
+                         ptr<float>(conv_state), cptr<T>(x), (int)x.stride(0),
+                         cptr<int>(seq_start), cptr<int>(seq_len),
+                         cptr<int>(seq_slot), cptr<int>(seq_pos0), C, taps);
+  });
+}
+
+void token_shift_mix(torch::Tensor out, torch::Tensor h, torch::Tensor mu,
+                     torch::Tensor prev_state, torch::Tensor tok_seq,
+                     torch::Tensor seq_start, torch::Tensor seq_len,
+                     torch::Tensor seq_slot, torch::Tensor seq_pos0) {
+  const int T_ = h.size(0), W = h.size(1), S = mu.size(0);
+  const int B = seq_start.size(0);
+  SEQ_CHECK(h.is_contiguous() && out.is_contiguous() &&
+                out.scalar_type() == h.scalar_type() && out.size(0) == S &&
+                out.size(1) == T_ && out.size(2) == W, "shift out");
+  SEQ_CHECK(mu.scalar_type() == torch::kFloat && mu.is_contiguous() &&
+                mu.size(1) == W, "shift mu");
+  SEQ_CHECK(prev_state.scalar_type() == torch::kFloat &&
+                prev_state.is_contiguous() && prev_state.size(1) == W,
+            "shift state");
+  check_seq(tok_seq, T_, "tok_seq");
+  check_seq(seq_len, B, "seq_len");
+  check_seq(seq_slot, B, "seq_slot");
+  check_seq(seq_pos0, B, "seq_pos0");
+  if (T_ == 0) return;
+  DISPATCH_ACT(h, {
+    hipLaunchKernelGGL(token_shift_mix_kernel<T>, dim3(T_), dim3(row_block(W)),
+                       0, cur_stream(), ptr<T>(out), cptr<T>(h),
+                       cptr<float>(mu), cptr<float>(prev_state),
+                       cptr<int>(tok_seq), cptr<int>(seq_start),
+                       cptr<int>(seq_slot), cptr<int>(seq_pos0), T_, W, S);
+    hipLaunchKernelGGL(shift_state_update_kernel<T>, dim3(B),
+                       dim3(row_block(W)), 0, cur_stream(),
+                       ptr<float>(prev_state), cptr<T>(h), cptr<int>(seq_start),
+                       cptr<int>(seq_len), cptr<int>(seq_slot), W);
+  });
+}
+
+void head_norm_gate(torch::Tensor out, torch::Tensor o, torch::Tensor w,
+                    int64_t w_stride, c10::optional<torch::Tensor> gate,
+                    int64_t gate_act, double eps) {
+  // o [T, H, dv] fp32; gate [T, >=H*dv] strided rows (column 0 = head 0)
+  const int T_ = o.size(0), H = o.size(1), dv = o.size(2);
+  SEQ_CHECK(o.scalar_type() == torch::kFloat && o.is_contiguous(), "head o");
+  SEQ_CHECK(out.is_contiguous() && out.numel() == o.numel(), "head out");
+  SEQ_CHECK(w.scalar_type() == torch::kFloat && w.is_contiguous() &&
+                w.numel() >= (H - 1) * w_stride + dv, "head weight");
+  SEQ_CHECK(gate_act == 0 || gate.has_value(), "gate missing");
+  if (gate)
+    SEQ_CHECK(gate->stride(1) == 1 && gate->size(0) == T_ &&
+                  gate->size(1) >= H * dv &&
+                  gate->scalar_type() == out.scalar_type(), "head gate");
+  if (T_ == 0) return;
+  DISPATCH_ACT(out, hipLaunchKernelGGL(
+      head_norm_gate_kernel<T>, dim3(T_, H), dim3(64), 0, cur_stream(),
+      ptr<T>(out), cptr<float>(o), cptr<float>(w), (int)w_stride,
+      gate ? cptr<T>(*gate) : (const T*)nullptr,
+      gate ? (int)gate->stride(0) : 0, (int)gate_act, (float)eps, H, dv););
+}
+
+void clamped_glu(torch::Tensor out, torch::Tensor gate_up, double limit,
+                 double alpha) {
+  const int64_t T_ = gate_up.size(0);
+  const int F = gate_up.size(1) / 2;
+  SEQ_CHECK(gate_up.is_contiguous() && out.is_contiguous() &&
+                out.size(0) == T_ && out.size(1) == F &&
+                out.scalar_type() == gate_up.scalar_type(), "glu shapes");
+  const int64_t n = T_ * F;
+  if (n == 0) return;
+  DISPATCH_ACT(out, hipLaunchKernelGGL(
+      clamped_glu_kernel<T>, dim3((n + 255) / 256), dim3(256), 0, cur_stream(),
+      ptr<T>(out), cptr<T>(gate_up), F, (float)limit, (float)alpha, n););
+}
+
+void dual_rmsnorm_mean(torch::Tensor out, torch::Tensor a, torch::Tensor b,
+                       torch::Tensor wa, torch::Tensor wb, double eps) {
+  const int T_ = a.size(0), W = a.size(1);
+  SEQ_CHECK(a.is_contiguous() && b.is_contiguous() && out.is_contiguous() &&
+                b.sizes() == a.sizes() && out.sizes() == a.sizes() &&
+                a.scalar_type() == b.scalar_type() &&
+                a.scalar_type() == out.scalar_type(), "merge shapes");
+  SEQ_CHECK(wa.scalar_type() == torch::kFloat && wa.numel() == W &&
+                wb.scalar_type() == torch::kFloat && wb.numel() == W,
+            "merge weights");
+  if (T_ == 0) return;
+  DISPATCH_ACT(out, hipLaunchKernelGGL(
+      dual_rmsnorm_mean_kernel<T>, dim3(T_), dim3(row_block(W)), 0,
+      cur_stream(), ptr<T>(out), cptr<T>(a), cptr<T>(b), cptr<float>(wa),
+      cptr<float>(wb), (float)eps, W););
+}
+
+void softcap_(torch::Tensor x, double cap) {
+  SEQ_CHECK(x.scalar_type() == torch::kFloat && x.is_contiguous(), "softcap");
+  const int64_t n = x.numel();
+  if (n == 0) return;
+  hipLaunchKernelGGL(softcap_kernel, dim3((n + 255) / 256), dim3(256), 0,
+                     cur_stream(), ptr<float>(x), (float)cap, n);
+}

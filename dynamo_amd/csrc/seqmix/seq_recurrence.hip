@@ -1,0 +1,442 @@
+// Matrix-state recurrences: gated delta rule, RWKV-style time mixing with
+// per-channel decay, and the mLSTM matrix memory. One workgroup owns a run
+// of value columns of one (sequence, head) state S [dk, dv] and walks the
+// sequence's rows of this step in order; a decoded token is a run of one.
+//
+// All three recurrences are independent per value column j: column j of S
+// is only ever combined with the token's key-side vectors. A thread keeps
+// R rows of one column in registers; KP threads (adjacent at lane distance
+// JW = 64 / KP) share a column and reduce their partial dot products with
+// lane shuffles. R <= RMAX and KP is a power of two, so dk <= RMAX * 64.
+// State is fp32 in HBM, loaded once per step and stored once.
+#include "seq_common.h"
+
+namespace {
+
+constexpr int RMAX = 32;
+
+struct SeqArgs {
+  const int* seq_start;
+  const int* seq_len;
+  const int* seq_slot;
+  const int* seq_pos0;
+};
+
+struct Geometry {
+  int KP, R, JW, NW, tiles;
+};
+
+inline Geometry geometry(int dk, int dv) {
+  Geometry g;
+  g.KP = 1;
+  while (g.KP * RMAX < dk) g.KP <<= 1;
+  TORCH_CHECK(g.KP <= 64, "seqmix: key size too large for the recurrence");
+  g.R = (dk + g.KP - 1) / g.KP;
+  g.JW = 64 / g.KP;
+  const int waves = (dv + g.JW - 1) / g.JW;
+  g.NW = waves < 4 ? waves : 4;
+  g.tiles = (waves + g.NW - 1) / g.NW;
+  return g;
+}
+
+// reduce over the KP lanes that share a column
+DEVINL float part_sum(float x, int JW) {
+  for (int off = JW; off < 64; off <<= 1) x += __shfl_xor(x, off, 64);
+  return x;
+}
+
+#define LOAD_STATE(S, base, fresh)                                    \
+  _Pragma("unroll") for (int r = 0; r < RMAX; r++) {                   \
+    const int row = part * R + r;                                      \
+    S[r] = (!fresh && r < R && row < dk && valid)                      \
+               ? base[(int64_t)row * dv + j] : 0.f;                    \
+  }
+#define STORE_STATE(S, base)                                          \
+  _Pragma("unroll") for (int r = 0; r < RMAX; r++) {                   \
+    const int row = part * R + r;                                      \
+    if (r < R && row < dk && valid) base[(int64_t)row * dv + j] = S[r]; \
+  }
+
+// ---------------------------------------------------------------------------
+// Gated delta rule. Per token: S <- g S; u = beta (v - S^T k);
+// S <- S + k u^T; o = S^T q. q and k arrive after the short convolution and
+// are made unit vectors here (q also scaled by qscale).
+template <typename T>
+__global__ void gated_delta_kernel(
+    float* __restrict__ out,          // [T, H, dv]
+    const float* __restrict__ qkv,    // [T, Cq + Ck + Cv] after conv + silu
+    const T* __restrict__ proj, int proj_stride, int off_b, int off_a,
+    const float* __restrict__ A_log, const float* __restrict__ dt_bias,
+    float* __restrict__ state,        // [slots, H, dk, dv]
+    SeqArgs sa, int H, int G, int dk, int dv, int KP, int R, float qscale,
+    float unit_eps) {
+  extern __shared__ float lds[];  // [2][dk]: unit k, scaled unit q
+  const int s = blockIdx.x, hh = blockIdx.y;
+  const int len = sa.seq_len[s];
+  if (len == 0) return;
+  const int start = sa.seq_start[s];
+  const bool fresh = sa.seq_pos0[s] == 0;
+  const int JW = 64 / KP;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int part = lane / JW;
+  const int nw = blockDim.x >> 6;
+  const int j = (blockIdx.z * nw + wave) * JW + (lane % JW);
+  const bool valid = j < dv;
+  const int kvh = hh / (H / G);
+  const int Cq = G * dk, Cc = 2 * G * dk + H * dv;
+  float* sbase = state + ((int64_t)sa.seq_slot[s] * H + hh) * dk * dv;
+  float* kl = lds;
+  float* ql = lds + dk;
+  float S[RMAX];
+  LOAD_STATE(S, sbase, fresh)
+  const float a_neg = -expf(A_log[hh]);
+  const float dtb = dt_bias[hh];
+
+  for (int t = start; t < start + len; t++) {
+    const float* row = qkv + (int64_t)t * Cc;
+    // every wave normalises redundantly; wave 0 publishes
+    float sq = 0.f, sk = 0.f;
+    for (int i = lane; i < dk; i += 64) {
+      const float qv = row[kvh * dk + i], kv = row[Cq + kvh * dk + i];
+      sq += qv * qv;
+      sk += kv * kv;
+    }
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    const float qn = qscale / sqrtf(sq + unit_eps);
+    const float kn = 1.f / sqrtf(sk + unit_eps);
+    __syncthreads();  // previous token's readers are done
+    for (int i = threadIdx.x; i < dk; i += blockDim.x) {
+      kl[i] = row[Cq + kvh * dk + i] * kn;
+      ql[i] = row[kvh * dk + i] * qn;
+    }
+    __syncthreads();
+    const float braw = to_f(proj[(int64_t)t * proj_stride + off_b + hh]);
+    const float araw = to_f(proj[(int64_t)t * proj_stride + off_a + hh]);
+    const float beta = sigmoid_f(braw);
+    const float g = expf(a_neg * softplus_f(araw + dtb));
+    const float vj = valid ? row[2 * Cq + hh * dv + j] : 0.f;
+    float dot = 0.f;
+#pragma unroll
+    for (int r = 0; r < RMAX; r++) {
+      const int rowi = part * R + r;
+      if (r < R && rowi < dk) {
+        S[r] *= g;
+        dot += S[r] * kl[rowi];
+      }
+    }
+    dot = part_sum(dot, JW);
+    const float u = beta * (vj - dot);
+    float o = 0.f;
+#pragma unroll
+    for (int r = 0; r < RMAX; r++) {
+      const int rowi = part * R + r;
+      if (r < R && rowi < dk) {
+        S[r] += kl[rowi] * u;
+        o += S[r] * ql[rowi];
+      }
+    }
+    o = part_sum(o, JW);
+    if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = o;
+  }
+  STORE_STATE(S, sbase)
+}
+
+// ---------------------------------------------------------------------------
+// RWKV-style time mixing. Per token, with w = exp(-exp(wraw + w0)):
+// o = (S + diag(u) k v^T)^T r; S <- diag(w) S + k v^T.
+template <typename T>
+__global__ void rwkv_kernel(
+    float* __restrict__ out,       // [T, H, d]
+    const T* __restrict__ r_, const T* __restrict__ k_,
+    const T* __restrict__ v_,      // [T, H*d] each
+    const T* __restrict__ wraw,    // [T, H*d]
+    const float* __restrict__ w0,  // [H*d]
+    const float* __restrict__ u,   // [H, d]
+    float* __restrict__ state,     // [slots, H, d, d]
+    SeqArgs sa, int H, int dk, int dv, int KP, int R) {
+  extern __shared__ float lds[];  // [3][dk]: r, k, w
+  const int s = blockIdx.x, hh = blockIdx.y;
+  const int len = sa.seq_len[s];
+  if (len == 0) return;
+  const int start = sa.seq_start[s];
+  const bool fresh = sa.seq_pos0[s] == 0;
+  const int JW = 64 / KP;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int part = lane / JW;
+  const int nw = blockDim.x >> 6;
+  const int j = (blockIdx.z * nw + wave) * JW + (lane % JW);
+  const bool valid = j < dv;
+  float* sbase = state + ((int64_t)sa.seq_slot[s] * H + hh) * dk * dv;
+  float* rl = lds;
+  float* kl = lds + dk;
+  float* wl = lds + 2 * dk;
+  float S[RMAX], U[RMAX];
+  LOAD_STATE(S, sbase, fresh)
+#pragma unroll
+  for (int r = 0; r < RMAX; r++) {
+    const int rowi = part * R + r;
+    U[r] = (r < R && rowi < dk) ? u[hh * dk + rowi] : 0.f;
+  }
+  const int HD = H * dk;
+  for (int t = start; t < start + len; t++) {
+    const int64_t base = (int64_t)t * HD + hh * dk;
+    __syncthreads();
+    for (int i = threadIdx.x; i < dk; i += blockDim.x) {
+      rl[i] = to_f(r_[base + i]);
+      kl[i] = to_f(k_[base + i]);
+      wl[i] = expf(-expf(to_f(wraw[base + i]) + w0[hh * dk + i]));
+    }
+    __syncthreads();
+    const float vj = valid ? to_f(v_[(int64_t)t * H * dv + hh * dv + j]) : 0.f;
+    float o = 0.f;
+#pragma unroll
+    for (int r = 0; r < RMAX; r++) {
+      const int rowi = part * R + r;
+      if (r < R && rowi < dk) {
+        const float kv = kl[rowi] * vj;
+        o += rl[rowi] * (S[r] + U[r] * kv);
+        S[r] = wl[rowi] * S[r] + kv;
+      }
+    }
+    o = part_sum(o, JW);
+    if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = o;
+  }
+  STORE_STATE(S, sbase)
+}
+
+// ---------------------------------------------------------------------------
+// mLSTM matrix memory with a stabiliser m that starts at 0.
+// i = cap tanh((iraw + ib) / cap); f = logsigmoid(cap tanh((fraw + fb) / cap))
+// m' = max(f + m, i); S <- e^(f+m-m') S + e^(i-m') k v^T; n likewise with k;
+// o = S^T q / (max(|n . q|, e^(-m')) + den_eps).
+template <typename T>
+__global__ void mlstm_kernel(
+    float* __restrict__ out,  // [T, H, dv]
+    const T* __restrict__ proj, int proj_stride, int off_q, int off_k,
+    int off_v, int off_i, int off_f, const float* __restrict__ i_bias,
+    const float* __restrict__ f_bias,
+    float* __restrict__ state_S,        // [slots, H, dk, dv]
+    const float* __restrict__ state_n,  // [slots, H, dk]
+    const float* __restrict__ state_m,  // [slots, H]
+    SeqArgs sa, int H, int dk, int dv, int KP, int R, float qscale, float cap,
+    float den_eps) {
+  extern __shared__ float lds[];  // [2][dk]: k, q
+  const int s = blockIdx.x, hh = blockIdx.y;
+  const int len = sa.seq_len[s];
+  if (len == 0) return;
+  const int start = sa.seq_start[s];
+  const bool fresh = sa.seq_pos0[s] == 0;
+  const int JW = 64 / KP;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int part = lane / JW;
+  const int nw = blockDim.x >> 6;
+  const int j = (blockIdx.z * nw + wave) * JW + (lane % JW);
+  const bool valid = j < dv;
+  const int slot = sa.seq_slot[s];
+  float* sbase = state_S + ((int64_t)slot * H + hh) * dk * dv;
+  const float* nbase = state_n + ((int64_t)slot * H + hh) * dk;
+  float* kl = lds;
+  float* ql = lds + dk;
+  float S[RMAX], N[RMAX];
+  LOAD_STATE(S, sbase, fresh)
+#pragma unroll
+  for (int r = 0; r < RMAX; r++) {
+    const int rowi = part * R + r;
+    N[r] = (!fresh && r < R && rowi < dk) ? nbase[rowi] : 0.f;
+  }
+  float m = fresh ? 0.f : state_m[slot * H + hh];
+  const float ib = i_bias[hh], fb = f_bias[hh];
+
+  for (int t = start; t < start + len; t++) {
+    const T* row = proj + (int64_t)t * proj_stride;
+    __syncthreads();
+    for (int i = threadIdx.x; i < dk; i += blockDim.x) {
+      kl[i] = to_f(row[off_k + hh * dk + i]);
+      ql[i] = to_f(row[off_q + hh * dk + i]) * qscale;
+    }
+    __syncthreads();
+    const float ig = cap * tanhf((to_f(row[off_i + hh]) + ib) / cap);
+    const float fg = logsigmoid_f(cap * tanhf((to_f(row[off_f + hh]) + fb) / cap));
+    const float mn = fmaxf(fg + m, ig);
+    const float a = expf(fg + m - mn), b = expf(ig - mn);
+    m = mn;
+    const float vj = valid ? to_f(row[off_v + hh * dv + j]) : 0.f;
+    float num = 0.f, nq = 0.f;
+#pragma unroll
+    for (int r = 0; r < RMAX; r++) {
+      const int rowi = part * R + r;
+      if (r < R && rowi < dk) {
+        const float bk = b * kl[rowi];
+        S[r] = a * S[r] + bk * vj;
+        N[r] = a * N[r] + bk;
+        num += S[r] * ql[rowi];
+        nq += N[r] * ql[rowi];
+      }
+    }
+    num = part_sum(num, JW);
+    nq = part_sum(nq, JW);
+    const float den = fmaxf(fabsf(nq), expf(-m)) + den_eps;
+    if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = num / den;
+  }
+  STORE_STATE(S, sbase)
+}
+
+// The normaliser n and stabiliser m are shared by every column tile of a
+// head, so the tiles above only read them; this pass, launched after, walks
+// the same gates once per (sequence, head) and stores the new n and m.
+template <typename T>
+__global__ void mlstm_nm_kernel(
+    const T* __restrict__ proj, int proj_stride, int off_k, int off_i,
+    int off_f, const float* __restrict__ i_bias,
+    const float* __restrict__ f_bias, float* __restrict__ state_n,
+    float* __restrict__ state_m, SeqArgs sa, int H, int dk, float cap) {
+  const int s = blockIdx.x, hh = blockIdx.y;
+  const int len = sa.seq_len[s];
+  if (len == 0) return;
+  const int start = sa.seq_start[s];
+  const bool fresh = sa.seq_pos0[s] == 0;
+  const int slot = sa.seq_slot[s];
+  float* nbase = state_n + ((int64_t)slot * H + hh) * dk;
+  float m0 = fresh ? 0.f : state_m[slot * H + hh];
+  const float ib = i_bias[hh], fb = f_bias[hh];
+  float m_end = m0;  // same on every thread; thread 0 owns row 0
+  for (int i = threadIdx.x; i < dk; i += blockDim.x) {
+    float n = fresh ? 0.f : nbase[i];
+    float m = m0;
+    for (int t = start; t < start + len; t++) {
+      const T* row = proj + (int64_t)t * proj_stride;
+      const float ig = cap * tanhf((to_f(row[off_i + hh]) + ib) / cap);
+      const float fg =
+          logsigmoid_f(cap * tanhf((to_f(row[off_f + hh]) + fb) / cap));
+      const float mn = fmaxf(fg + m, ig);
+      n = expf(fg + m - mn) * n + expf(ig - mn) * to_f(row[off_k + hh * dk + i]);
+      m = mn;
+    }
+    nbase[i] = n;
+    m_end = m;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) state_m[slot * H + hh] = m_end;
+}
+
+SeqArgs seq_args(const torch::Tensor& seq_start, const torch::Tensor& seq_len,
+                 const torch::Tensor& seq_slot, const torch::Tensor& seq_pos0,
+                 int64_t slots) {
+  const int64_t B = seq_start.size(0);
+  for (const torch::Tensor* t : {&seq_start, &seq_len, &seq_slot, &seq_pos0})
+    TORCH_CHECK(t->scalar_type() == torch::kInt && t->is_contiguous() &&
+                    t->numel() >= B && t->is_cuda(),
+                "seqmix: sequence descriptors must be int32 device tensors");
+  (void)slots;
+  return SeqArgs{cptr<int>(seq_start), cptr<int>(seq_len), cptr<int>(seq_slot),
+                 cptr<int>(seq_pos0)};
+}
+
+}  // namespace
+
+void gated_delta_rule(torch::Tensor out, torch::Tensor qkv, torch::Tensor proj,
+                      int64_t off_b, int64_t off_a, torch::Tensor A_log,
+                      torch::Tensor dt_bias, torch::Tensor state,
+                      torch::Tensor seq_start, torch::Tensor seq_len,
+                      torch::Tensor seq_slot, torch::Tensor seq_pos0,
+                      int64_t G, double qscale, double unit_eps) {
+  const int T_ = out.size(0), H = out.size(1), dv = out.size(2);
+  const int dk = state.size(2);
+  SEQ_CHECK(out.scalar_type() == torch::kFloat && out.is_contiguous(), "out");
+  SEQ_CHECK(state.scalar_type() == torch::kFloat && state.is_contiguous() &&
+                state.size(1) == H && state.size(3) == dv, "delta state");
+  SEQ_CHECK(G >= 1 && H % G == 0, "delta head grouping");
+  SEQ_CHECK(qkv.scalar_type() == torch::kFloat && qkv.is_contiguous() &&
+                qkv.size(0) == T_ && qkv.size(1) == 2 * G * dk + H * dv,
+            "delta qkv");
+  SEQ_CHECK(proj.stride(1) == 1 && proj.size(0) == T_ &&
+                off_b + H <= proj.size(1) && off_a + H <= proj.size(1),
+            "delta gates");
+  SEQ_CHECK(A_log.scalar_type() == torch::kFloat && A_log.numel() == H &&
+                dt_bias.scalar_type() == torch::kFloat && dt_bias.numel() == H,
+            "delta decay parameters");
+  const int B = seq_start.size(0);
+  if (T_ == 0 || B == 0) return;
+  SeqArgs sa = seq_args(seq_start, seq_len, seq_slot, seq_pos0, state.size(0));
+  Geometry g = geometry(dk, dv);
+  DISPATCH_ACT(proj, hipLaunchKernelGGL(
+      gated_delta_kernel<T>, dim3(B, H, g.tiles), dim3(g.NW * 64),
+      2 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<float>(qkv),
+      cptr<T>(proj), (int)proj.stride(0), (int)off_b, (int)off_a,
+      cptr<float>(A_log), cptr<float>(dt_bias), ptr<float>(state), sa, H,
+      (int)G, dk, dv, g.KP, g.R, (float)qscale, (float)unit_eps););
+}
+
+void rwkv_time_mix(torch::Tensor out, torch::Tensor r, torch::Tensor k,
+                   torch::Tensor v, torch::Tensor wraw, torch::Tensor w0,
+                   torch::Tensor u, torch::Tensor state,
+                   torch::Tensor seq_start, torch::Tensor seq_len,
+                   torch::Tensor seq_slot, torch::Tensor seq_pos0) {
+  const int T_ = out.size(0), H = out.size(1), dv = out.size(2);
+  const int dk = state.size(2);
+  SEQ_CHECK(out.scalar_type() == torch::kFloat && out.is_contiguous(), "out");
+  SEQ_CHECK(state.scalar_type() == torch::kFloat && state.is_contiguous() &&
+                state.size(1) == H && state.size(3) == dv, "rwkv state");
+  for (const torch::Tensor* t : {&r, &k, &wraw})
+    SEQ_CHECK(t->is_contiguous() && t->size(0) == T_ && t->size(1) == H * dk &&
+                  t->scalar_type() == r.scalar_type(), "rwkv r/k/w");
+  SEQ_CHECK(v.is_contiguous() && v.size(0) == T_ && v.size(1) == H * dv &&
+                v.scalar_type() == r.scalar_type(), "rwkv v");
+  SEQ_CHECK(w0.scalar_type() == torch::kFloat && w0.numel() == H * dk &&
+                u.scalar_type() == torch::kFloat && u.numel() == H * dk &&
+                w0.is_contiguous() && u.is_contiguous(), "rwkv w0/u");
+  const int B = seq_start.size(0);
+  if (T_ == 0 || B == 0) return;
+  SeqArgs sa = seq_args(seq_start, seq_len, seq_slot, seq_pos0, state.size(0));
+  Geometry g = geometry(dk, dv);
+  DISPATCH_ACT(r, hipLaunchKernelGGL(
+      rwkv_kernel<T>, dim3(B, H, g.tiles), dim3(g.NW * 64),
+      3 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(r),
+      cptr<T>(k), cptr<T>(v), cptr<T>(wraw), cptr<float>(w0), cptr<float>(u),
+      ptr<float>(state), sa, H, dk, dv, g.KP, g.R););
+}
+
+void mlstm_memory(torch::Tensor out, torch::Tensor proj, int64_t off_q,
+                  int64_t off_k, int64_t off_v, int64_t off_i, int64_t off_f,
+                  torch::Tensor i_bias, torch::Tensor f_bias,
+                  torch::Tensor state_S, torch::Tensor state_n,
+                  torch::Tensor state_m, torch::Tensor seq_start,
+                  torch::Tensor seq_len, torch::Tensor seq_slot,
+                  torch::Tensor seq_pos0, double qscale, double cap,
+                  double den_eps) {
+  const int T_ = out.size(0), H = out.size(1), dv = out.size(2);
+  const int dk = state_S.size(2);
+  SEQ_CHECK(out.scalar_type() == torch::kFloat && out.is_contiguous(), "out");
+  SEQ_CHECK(state_S.scalar_type() == torch::kFloat && state_S.is_contiguous() &&
+                state_S.size(1) == H && state_S.size(3) == dv, "mlstm S");
+  SEQ_CHECK(state_n.scalar_type() == torch::kFloat && state_n.is_contiguous() &&
+                state_n.size(0) == state_S.size(0) && state_n.size(1) == H &&
+                state_n.size(2) == dk, "mlstm n");
+  SEQ_CHECK(state_m.scalar_type() == torch::kFloat && state_m.is_contiguous() &&
+                state_m.size(0) == state_S.size(0) && state_m.size(1) == H,
+            "mlstm m");
+  const int64_t P = proj.size(1);
+  SEQ_CHECK(proj.stride(1) == 1 && proj.size(0) == T_ && off_q + H * dk <= P &&
+                off_k + H * dk <= P && off_v + H * dv <= P && off_i + H <= P &&
+                off_f + H <= P, "mlstm projections");
+  SEQ_CHECK(i_bias.scalar_type() == torch::kFloat && i_bias.numel() == H &&
+                f_bias.scalar_type() == torch::kFloat && f_bias.numel() == H,
+            "mlstm biases");
+  const int B = seq_start.size(0);
+  if (T_ == 0 || B == 0) return;
+  SeqArgs sa = seq_args(seq_start, seq_len, seq_slot, seq_pos0, state_S.size(0));
+  Geometry g = geometry(dk, dv);
+  DISPATCH_ACT(proj, hipLaunchKernelGGL(
+      mlstm_kernel<T>, dim3(B, H, g.tiles), dim3(g.NW * 64),
+      2 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(proj),
+      (int)proj.stride(0), (int)off_q, (int)off_k, (int)off_v, (int)off_i,
+      (int)off_f, cptr<float>(i_bias), cptr<float>(f_bias),
+      ptr<float>(state_S), ptr<float>(state_n), ptr<float>(state_m), sa, H, dk,
+      dv, g.KP, g.R, (float)qscale, (float)cap, (float)den_eps);
+    hipLaunchKernelGGL(
+      mlstm_nm_kernel<T>, dim3(B, H), dim3(dk < 64 ? 64 : (dk > 256 ? 256 : (dk + 63) / 64 * 64)),
+      0, cur_stream(), cptr<T>(proj), (int)proj.stride(0), (int)off_k,
+      (int)off_i, (int)off_f, cptr<float>(i_bias), cptr<float>(f_bias),
+      ptr<float>(state_n), ptr<float>(state_m), sa, H, dk, (float)cap););
+}

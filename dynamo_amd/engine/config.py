@@ -16,7 +16,7 @@ from typing import Optional
 @dataclass
 class ModelConfig:
     name: str = "llama-3-8b"
-    arch: str = "llama"            # llama | opt | mixtral | qwen2
+    arch: str = "llama"            # llama | opt | mixtral | qwen2 | bolatar
     hidden_size: int = 4096
     intermediate_size: int = 14336
     num_layers: int = 32
@@ -39,6 +39,11 @@ class ModelConfig:
     learned_pos_emb: bool = False
     # qwen2-style QKV bias
     attn_bias: bool = False
+    # layer-list models (bolatar): one dict per layer with its mixer type,
+    # mixer sizes and feed-forward, as in the checkpoint's config.json
+    layer_specs: Optional[list] = None
+    embed_scale: float = 1.0       # multiplies token embeddings
+    logit_softcap: float = 0.0     # cap * tanh(logits / cap); 0 = off
     # local HF checkpoint dir to load real weights from ("" = random init)
     weights_path: str = ""
 
@@ -110,6 +115,25 @@ PRESETS = {
         intermediate_size=256, num_layers=2, num_q_heads=4, num_kv_heads=2,
         head_dim=32, vocab_size=512, max_position=2048, rope_theta=10000.0,
         num_experts=4, num_experts_per_tok=2),
+    # layer-list model: every mixer kind once, small odd sizes
+    "tiny-bolatar": ModelConfig(
+        name="tiny-bolatar", arch="bolatar", hidden_size=96, vocab_size=160,
+        max_position=512, num_layers=3, rms_eps=1e-5, learned_pos_emb=True,
+        embed_scale=2.0, logit_softcap=20.0, intermediate_size=0,
+        num_q_heads=1, num_kv_heads=1, head_dim=1,
+        layer_specs=[
+            {"type": "parallel", "mixer": {
+                "left": {"heads": 6, "kv_heads": 3, "dim": 24, "vdim": 40,
+                         "scale": 0.2, "q_temp": {"coef": 0.2, "every": 16}},
+                "right": {"heads": 3, "dim": 32}},
+             "mlp": {"kind": "dense", "ff": 144, "limit": 3.0}},
+            {"type": "delta", "mixer": {"heads": 4, "kv_heads": 2, "dim": 24,
+                                        "vdim": 16, "conv": 3},
+             "mlp": None},
+            {"type": "mlstm", "mixer": {"heads": 2, "dim": 16, "vdim": 48,
+                                        "gate_cap": 10.0},
+             "mlp": {"kind": "dense", "ff": 120, "limit": 2.5}},
+        ]),
 }
 
 

@@ -50,9 +50,20 @@ class ForwardPassMetrics:
 class LLMEngine:
     def __init__(self, cfg: EngineConfig, tp: Optional[TPContext] = None,
                  seed: int = 0, runner=None, weight_pool=None):
-        self.cfg = cfg
         self.runner = (runner if runner is not None
                        else ModelRunner(cfg, tp, seed, weight_pool=weight_pool))
+        # recurrent state cannot be rebuilt from cached pages, so a model
+        # that carries any runs without prefix reuse and without the
+        # host/disk tiers; each running sequence owns one state slot
+        self.state_slots = None
+        sp = getattr(self.runner, "state_pool", None)
+        if sp is not None:
+            import dataclasses
+            from .state_cache import SlotAllocator
+            cfg = dataclasses.replace(cfg, enable_prefix_caching=False,
+                                      host_cache_pages=0)
+            self.state_slots = SlotAllocator(sp.num_slots)
+        self.cfg = cfg
         self.alloc = PageAllocator(self.runner.num_pages, cfg.page_size,
                                    cfg.enable_prefix_caching)
         self.host_tier = None
@@ -65,7 +76,7 @@ class LLMEngine:
                                         object_dir=cfg.object_cache_dir,
                                         policy=cfg.host_cache_policy)
             self.alloc.host_tier = self.host_tier
-        self.scheduler = Scheduler(cfg, self.alloc)
+        self.scheduler = Scheduler(cfg, self.alloc, self.state_slots)
         self.requests: Dict[str, Request] = {}
         self.step_count = 0
         self.kv_events: List[KvEvent] = []
@@ -204,6 +215,7 @@ class LLMEngine:
                     req.finish_reason = reason
                     req.finish_time = time.monotonic()
                     self.scheduler.running.remove(req)
+                    self.scheduler._release_state(req)
                     self._held[req.req_id] = req
                 else:
                     self._finish(req, reason)
@@ -266,6 +278,7 @@ class LLMEngine:
                     req.finish_reason = reason
                     req.finish_time = time.monotonic()
                     self.scheduler.running.remove(req)
+                    self.scheduler._release_state(req)
                     self._held[req.req_id] = req
                 else:
                     self._finish(req, reason)
@@ -307,6 +320,71 @@ class LLMEngine:
             total_kv_pages=self.alloc.num_pages,
         )
         return outputs
+
+    # ------------------------------------------------------------------
+    def replay_step(self, entries, end=()):
+        """Run one step of a recorded schedule instead of the scheduler's
+        own choice: `entries` is [(req_id, next_tokens, want)], where `want`
+        lists the places among next_tokens whose logits are returned (fp32
+        [n_wanted, vocab], in entry order). A request is admitted at its
+        first entry (pages and a state slot from the engine's allocators)
+        and released when named in `end`. All entries run as one batch
+        through the same forward path as step(): single next tokens of
+        started requests as decodes, longer portions as prefill chunks.
+        Nothing is sampled and nothing is preempted - a schedule that does
+        not fit the pool raises MemoryError."""
+        from .kv_cache import SequenceKV
+        from .scheduler import ScheduledSeq, SchedulerOutput
+        sched = SchedulerOutput()
+        items = []
+        for req_id, tokens, want in entries:
+            req = self.requests.get(req_id)
+            if req is None:
+                req = Request(req_id, [], SamplingParams(max_tokens=0))
+                req.kv = SequenceKV(self.alloc, self.cfg.block_salt)
+                if len(self.scheduler.running) >= self.cfg.max_num_seqs or \
+                        not self.scheduler._take_state(req):
+                    raise MemoryError("no free sequence slot")
+                req.state = ReqState.RUNNING
+                self.requests[req_id] = req
+                self.scheduler.running.append(req)
+            n = len(tokens)
+            if n == 0:
+                continue
+            req.prompt_tokens.extend(int(t) for t in tokens)
+            if req.total_len > self.cfg.max_model_len:
+                raise ValueError(f"{req_id} exceeds max_model_len")
+            req.kv.ensure_capacity(req.num_computed + n)
+            ss = ScheduledSeq(req, n, False)
+            decode = n == 1 and req.num_computed > 0
+            (sched.decodes if decode else sched.prefills).append(ss)
+            items.append((ss, decode, list(want)))
+        # rows of the flat batch: decodes first, then prefill chunks
+        base, row = {}, len(sched.decodes)
+        for i, ss in enumerate(sched.decodes):
+            base[id(ss)] = i
+        for ss in sched.prefills:
+            base[id(ss)] = row
+            row += ss.n_new
+        rows = [base[id(ss)] + w for ss, _d, want in items for w in want]
+        logits = None
+        if not sched.is_empty:
+            if self.graph_runner is not None:
+                self.graph_runner.dirty = True
+                self._last_sampled = None
+            self.step_count += 1
+            logits = self.runner.forward_logits(sched, rows)
+            for ss in sched.seqs:
+                ss.req.num_computed += ss.n_new
+                if self.cfg.enable_prefix_caching:
+                    ss.req.kv.commit_full_pages(ss.req.all_tokens,
+                                                ss.req.num_computed)
+        for req_id in end:
+            req = self.requests.pop(req_id, None)
+            if req is not None:
+                self._finish(req, "replay_end")
+        self.kv_events.extend(self.alloc.drain_events())
+        return logits
 
     def _finish(self, req: Request, reason: str):
         # commit full pages before release so prefix cache retains them

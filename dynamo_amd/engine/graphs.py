@@ -41,6 +41,12 @@ class GraphRunner:
         self.slot_mapping = torch.zeros(B, dtype=torch.int64, device=dev)
         self.page_table = torch.zeros(B, self.max_pages, dtype=torch.int32,
                                       device=dev)
+        # models with recurrent mixers: one single-token span per row
+        self.seq_model = bool(getattr(runner, "seq_model", False))
+        if self.seq_model:
+            self.seq_rows = torch.arange(B, dtype=torch.int32, device=dev)
+            self.seq_len = torch.zeros(B, dtype=torch.int32, device=dev)
+            self.seq_slot = torch.zeros(B, dtype=torch.int32, device=dev)
         V = cfg.model.vocab_size
         self.logits = torch.empty(B, V, dtype=torch.float32, device=dev)
         self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
@@ -52,6 +58,17 @@ class GraphRunner:
 
     # ------------------------------------------------------------------
     def _meta(self, bc: int) -> AttnMetadata:
+        meta = self._attn_meta(bc)
+        if self.seq_model:
+            from dynamo_amd.ops.seq import SeqBatch
+            meta.seq_batch = SeqBatch(
+                tok_seq=self.seq_rows[:bc], seq_start=self.seq_rows[:bc],
+                seq_len=self.seq_len[:bc], seq_slot=self.seq_slot[:bc],
+                seq_pos0=self.positions[:bc], page_table=self.page_table[:bc])
+            meta.state_pool = self.runner.state_pool
+        return meta
+
+    def _attn_meta(self, bc: int) -> AttnMetadata:
         return AttnMetadata(
             slot_mapping=self.slot_mapping[:bc],
             positions=self.positions[:bc],
@@ -114,6 +131,12 @@ class GraphRunner:
         if n < self.max_batch:
             self.ctx_lens[n:].fill_(0)
             self.slot_mapping[n:].fill_(-1)
+        if self.seq_model:
+            # pad rows are empty spans: no state is read or written
+            self.seq_len[:n].fill_(1)
+            self.seq_len[n:].fill_(0)
+            self.seq_slot[:n].copy_(torch.tensor(
+                [r.state_slot for r in reqs], dtype=torch.int32))
         self.dirty = False
         self._first_after_rebuild = True
 

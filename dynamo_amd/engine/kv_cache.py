@@ -233,7 +233,11 @@ class KVCachePool:
     def __init__(self, num_layers: int, num_pages: int, num_kv_heads: int,
                  page_size: int, head_dim: int, device: str,
                  dtype=torch.bfloat16, shm_export: bool = False,
-                 v_transposed: bool = False):
+                 v_transposed: bool = False, layer_shapes=None):
+        if layer_shapes is not None:
+            self._init_per_layer(layer_shapes, num_pages, page_size, device,
+                                 dtype)
+            return
         # v_transposed: V pages are stored d-major; vcache() views the same
         # storage as [P, Hkv, hd, ps] (page bytes and transfer granularity
         # are unchanged - copies and exports stay layout-agnostic)
@@ -270,6 +274,51 @@ class KVCachePool:
             self.buffer = torch.zeros(self.shape, dtype=dtype, device=device)
         self.nbytes = nbytes
 
+    def _init_per_layer(self, layer_shapes, num_pages, page_size, device,
+                        dtype):
+        """Pool for models whose layers differ: layer_shapes[i] is
+        (kv_heads, key_dim, value_dim), or None for a layer that caches
+        nothing. Still one allocation; layer i's K view is
+        [P, kv_heads, ps, key_dim] and its V view [P, kv_heads, ps,
+        value_dim]. Page ids are shared by all layers, as in the uniform
+        pool. Not exported over IPC (no disaggregated serving for these
+        models: their recurrent state would have to move too)."""
+        self.v_transposed = False
+        self.layer_shapes = list(layer_shapes)
+        self.num_pages = num_pages
+        self.page_size = page_size
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.shm_path = None
+        self.shape = None
+        offs, total = [], 0
+        for sh in self.layer_shapes:
+            if sh is None:
+                offs.append(None)
+                continue
+            g, dk, dv = sh
+            nk = num_pages * g * page_size * dk
+            nv = num_pages * g * page_size * dv
+            offs.append((total, nk, total + nk, nv))
+            total += nk + nv
+        self.buffer = torch.zeros(max(total, 1), dtype=dtype, device=device)
+        self._views = []
+        for sh, o in zip(self.layer_shapes, offs):
+            if sh is None:
+                self._views.append(None)
+                continue
+            g, dk, dv = sh
+            k0, nk, v0, nv = o
+            self._views.append((
+                self.buffer[k0:k0 + nk].view(num_pages, g, page_size, dk),
+                self.buffer[v0:v0 + nv].view(num_pages, g, page_size, dv)))
+        self.nbytes = total * self.buffer.element_size()
+
+    @staticmethod
+    def page_bytes_per_layer_shapes(layer_shapes, page_size, elem_size):
+        return sum(sh[0] * page_size * (sh[1] + sh[2]) * elem_size
+                   for sh in layer_shapes if sh is not None)
+
     def __del__(self):  # pragma: no cover
         if getattr(self, "shm_path", None):
             import os
@@ -279,9 +328,13 @@ class KVCachePool:
                 pass
 
     def kcache(self, layer: int) -> torch.Tensor:
+        if self.shape is None:
+            return self._views[layer][0]
         return self.buffer[layer, 0]
 
     def vcache(self, layer: int) -> torch.Tensor:
+        if self.shape is None:
+            return self._views[layer][1]
         v = self.buffer[layer, 1]
         if self.v_transposed:
             _, _, P, hkv, ps, hd = self.shape

@@ -43,6 +43,15 @@ class ModelRunner:
                 "loaded %d checkpoint tensors from %s", n, m.weights_path)
         self.hkv_local = max(1, m.num_kv_heads // self.tp.size)
         self.hq_local = m.num_q_heads // self.tp.size
+        # layer-list models declare per-layer cache shapes and recurrent
+        # state; uniform-attention models have neither hook
+        self.seq_model = bool(getattr(self.model, "needs_seq_batch", False))
+        self.state_pool = None
+        self.max_pages_per_seq = ((cfg.max_model_len + cfg.page_size - 1)
+                                  // cfg.page_size)
+        if self.seq_model:
+            self._init_seq_model()
+            return
 
         num_pages = cfg.kv_pool_pages or self._auto_pages()
         # resolve the V-page layout against the LOCAL (TP-sharded) head
@@ -63,10 +72,32 @@ class ModelRunner:
                 cfg.max_num_seqs, self.hq_local, m.head_dim,
                 cfg.max_model_len, self.device)
 
-    def _auto_pages(self) -> int:
+    def _init_seq_model(self):
+        """Per-layer paged cache + slot-addressed recurrent state."""
+        from .state_cache import RecurrentStatePool
+        cfg = self.cfg
+        if cfg.kv_cache_dtype != "auto":
+            raise ValueError("layer-list models keep the cache in the "
+                             "compute dtype")
+        kv_shapes = self.model.kv_layer_shapes()
+        esize = torch.tensor([], dtype=self.dtype).element_size()
+        page_bytes = KVCachePool.page_bytes_per_layer_shapes(
+            kv_shapes, cfg.page_size, esize)
+        self.state_pool = RecurrentStatePool(self.model.state_layer_shapes(),
+                                             cfg.max_num_seqs, self.device)
+        num_pages = cfg.kv_pool_pages or self._auto_pages(max(1, page_bytes))
+        self.v_transposed = False
+        self.kv_pool = KVCachePool(0, num_pages, 0, cfg.page_size, 0,
+                                   cfg.device, self.dtype,
+                                   layer_shapes=kv_shapes)
+        self.num_pages = num_pages
+        self.decode_scratch = None
+
+    def _auto_pages(self, page_bytes: int = 0) -> int:
         m = self.cfg.model
-        page_bytes = (m.num_layers * 2 * self.hkv_local * self.cfg.page_size
-                      * m.head_dim * 2)
+        page_bytes = page_bytes or (
+            m.num_layers * 2 * self.hkv_local * self.cfg.page_size
+            * m.head_dim * 2)
         if self.device.type == "cuda":
             free, _total = torch.cuda.mem_get_info(self.device)
             budget = int(free * self.cfg.gpu_mem_fraction) - (2 << 30)
@@ -164,6 +195,9 @@ class ModelRunner:
             logits_rows=torch.tensor(logits_rows, dtype=torch.int64).to(dev, non_blocking=True),
             v_transposed=self.v_transposed,
         )
+        if self.seq_model:
+            meta.seq_batch = self._seq_batch(sched, dec_tables + pf_tables)
+            meta.state_pool = self.state_pool
         if embeds_rows:
             meta.embeds_rows = torch.tensor(embeds_rows, dtype=torch.int64,
                                             device=dev)
@@ -173,6 +207,47 @@ class ModelRunner:
             meta.prefill_tiles = ops.build_prefill_tiles(q_len, dev, rows)
         input_ids = torch.tensor(tokens, dtype=torch.int32).to(dev, non_blocking=True)
         return input_ids, meta
+
+    def _seq_batch(self, sched: SchedulerOutput, tables):
+        """Sequence spans of the flat batch (decodes, then prefill chunks):
+        rows, state slot and first position of each, plus one page table
+        for all of them."""
+        from dynamo_amd.ops.seq import SeqBatch
+        dev = self.device
+        spans, tok_seq = [], []
+        row = 0
+        for ss in sched.decodes + sched.prefills:
+            r = ss.req
+            if r.state_slot is None:
+                raise RuntimeError(f"{r.req_id} runs without a state slot")
+            spans.append((row, ss.n_new, r.state_slot, r.num_computed))
+            tok_seq.extend([len(spans) - 1] * ss.n_new)
+            row += ss.n_new
+        maxp = max([len(t) for t in tables] + [1])
+        pt = torch.zeros(len(tables), maxp, dtype=torch.int32)
+        for i, t in enumerate(tables):
+            pt[i, :len(t)] = torch.tensor(t, dtype=torch.int32)
+        cols = torch.tensor(spans, dtype=torch.int32).reshape(-1, 4).t(
+            ).contiguous().to(dev, non_blocking=True)
+        return SeqBatch(
+            tok_seq=torch.tensor(tok_seq, dtype=torch.int32).to(
+                dev, non_blocking=True),
+            seq_start=cols[0], seq_len=cols[1], seq_slot=cols[2],
+            seq_pos0=cols[3], page_table=pt.to(dev, non_blocking=True),
+            host=spans)
+
+    # ------------------------------------------------------------------
+    @torch.inference_mode()
+    def forward_logits(self, sched: SchedulerOutput, rows: List[int]):
+        """One forward over `sched`; fp32 logits of the given rows of the
+        flat batch (decodes first, then prefill chunks). The same path as
+        execute() up to sampling - used to replay recorded schedules."""
+        input_ids, meta = self.prepare(sched)
+        hidden = self.model.forward(input_ids, self.kv_pool, meta)
+        if not rows:
+            return torch.empty(0, self.cfg.model.vocab_size)
+        idx = torch.tensor(rows, dtype=torch.int64).to(self.device)
+        return self.model.compute_logits(hidden[idx])
 
     # ------------------------------------------------------------------
     @torch.inference_mode()

@@ -74,6 +74,8 @@ class Request:
         # of token-table embeddings (reference: preprocessor.rs:2248 media
         # + encode-worker embeddings spliced into the P/D request)
         self.embed_spans = None
+        # recurrent-state slot (models with state-carrying mixers)
+        self.state_slot: Optional[int] = None
 
     @property
     def has_embeds(self) -> bool:
@@ -124,9 +126,13 @@ class SchedulerOutput:
 
 
 class Scheduler:
-    def __init__(self, cfg: EngineConfig, allocator: PageAllocator):
+    def __init__(self, cfg: EngineConfig, allocator: PageAllocator,
+                 state_slots=None):
         self.cfg = cfg
         self.alloc = allocator
+        # SlotAllocator when the model carries recurrent state: a sequence
+        # holds one slot from admission until it finishes or is preempted
+        self.state_slots = state_slots
         self.waiting: List[Request] = []
         self.running: List[Request] = []
 
@@ -157,6 +163,7 @@ class Scheduler:
             self.running.pop(i)
             victim.kv.release()
             victim.kv = None
+            self._release_state(victim)
             victim.num_computed = 0
             victim.num_preemptions += 1
             victim.state = ReqState.WAITING
@@ -195,6 +202,7 @@ class Scheduler:
                 self.running.remove(req)
                 req.kv.release()
                 req.kv = None
+                self._release_state(req)
                 req.num_computed = 0
                 req.num_preemptions += 1
                 req.state = ReqState.WAITING
@@ -222,6 +230,8 @@ class Scheduler:
                 break
             if not self._ensure_pages(req, req.num_computed + n, out):
                 break
+            if not self._take_state(req):
+                break       # every slot is held by a running sequence
             self.waiting.pop(0)
             req.state = ReqState.RUNNING
             self.running.append(req)
@@ -240,6 +250,17 @@ class Scheduler:
             budget -= n
 
         return out
+
+    def _take_state(self, req: Request) -> bool:
+        if self.state_slots is None or req.state_slot is not None:
+            return True
+        req.state_slot = self.state_slots.alloc(req.req_id)
+        return req.state_slot is not None
+
+    def _release_state(self, req: Request):
+        if self.state_slots is not None and req.state_slot is not None:
+            self.state_slots.release(req.state_slot)
+        req.state_slot = None
 
     def _order_waiting(self):
         pol = getattr(self.cfg, "queue_policy", "fcfs")
@@ -260,6 +281,7 @@ class Scheduler:
         if req.kv is not None:
             req.kv.release()
             req.kv = None
+        self._release_state(req)
         if req in self.running:
             self.running.remove(req)
 

@@ -47,6 +47,10 @@ class AttnMetadata:
     inputs_embeds: Optional[torch.Tensor] = None       # [Te, hidden]
     # V pages stored d-major (see EngineConfig.kv_v_layout)
     v_transposed: bool = False
+    # models with recurrent mixers: per-sequence spans/slots of this batch
+    # (ops.seq.SeqBatch) and the engine's RecurrentStatePool
+    seq_batch: Optional[object] = None
+    state_pool: Optional[object] = None
 
 
 def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:

@@ -39,6 +39,9 @@ def config_from_hf(path: str) -> ModelConfig:
     """Build a ModelConfig from an HF checkpoint dir's config.json."""
     with open(os.path.join(path, "config.json")) as f:
         hf = json.load(f)
+    if str(hf.get("architecture", "")).lower() == "bolatar":
+        from dynamo_amd.models.bolatar import config_from_json
+        return config_from_json(hf, os.path.basename(os.path.normpath(path)))
     archs = [a.lower() for a in hf.get("architectures", [])]
     if any("mixtral" in a for a in archs):
         arch = "mixtral"
@@ -88,6 +91,9 @@ def _shard(full: torch.Tensor, dim: int, n: int, idx: int) -> torch.Tensor:
 def load_weights(model, path: str, strict: bool = True) -> int:
     """Load an HF checkpoint dir into a built model (in place). Returns the
     number of checkpoint tensors consumed."""
+    if hasattr(model, "load_checkpoint"):
+        # layer-list models map their own tensor names
+        return model.load_checkpoint(path)
     cfg = model.cfg
     tp = model.tp
     hd = cfg.head_dim

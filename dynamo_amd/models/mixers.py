@@ -1,0 +1,322 @@
+"""Token mixers beyond rotary softmax attention: recurrent matrix-state
+mixers with a slot-addressed fp32 state, and softmax attention with a
+distance bias / query temperature / value norm over the paged cache.
+
+Every mixer takes the normed hidden rows h [T, W] of the engine's flat
+batch and a `MixContext` (sequence spans, state tensors of its layer, cache
+views) and returns [T, W] in the activation dtype. Constants of a mechanism
+are constructor parameters; sizes come from the weights' shapes.
+
+Big projections are one fused GEMM where the inputs allow it (hipBLASLt via
+F.linear); what follows them runs in the HIP kernels of ops.seq. Small
+per-channel parameters are kept in fp32.
+
+Each class declares what the engine must hold for it:
+  state_shapes()  per-slot shapes of its recurrent state tensors (fp32)
+  kv_shape()      (kv_heads, key_dim, value_dim) of its paged cache, or None
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, List, Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+
+from dynamo_amd.ops import seq as sops
+
+
+@dataclass
+class MixContext:
+    sb: "sops.SeqBatch"
+    positions: torch.Tensor                 # [T] int32
+    slot_mapping: torch.Tensor              # [T] int64 cache slots
+    states: List[torch.Tensor]              # this layer's state tensors
+    kcache: Optional[torch.Tensor] = None   # [P, G, ps, dk]
+    vcache: Optional[torch.Tensor] = None   # [P, G, ps, dv]
+
+
+class _Init:
+    """Seeded random weights (benchmarks and tests run on random models)."""
+
+    def __init__(self, device, dtype, gen):
+        self.device, self.dtype, self.gen = device, dtype, gen
+
+    def mat(self, out, inp, std=None):
+        std = inp ** -0.5 if std is None else std
+        w = torch.randn(out, inp, generator=self.gen, dtype=torch.float32) * std
+        return w.to(self.dtype).to(self.device)
+
+    def vec(self, shape, lo, hi):
+        if isinstance(shape, int):
+            shape = (shape,)
+        w = torch.rand(*shape, generator=self.gen, dtype=torch.float32)
+        return (lo + (hi - lo) * w).to(self.device)
+
+
+Getter = Callable[[str], torch.Tensor]
+
+
+def _put(dst: torch.Tensor, src: torch.Tensor):
+    if tuple(dst.shape) != tuple(src.shape):
+        raise ValueError(f"shape mismatch {tuple(dst.shape)} vs "
+                         f"{tuple(src.shape)}")
+    with torch.no_grad():
+        dst.copy_(src.to(dst.dtype))
+
+
+class GatedDeltaMixer(torch.nn.Module):
+    """Gated delta rule with short causal convolutions on q, k, v.
+
+    S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, with unit
+    q/k per head, q scaled by dk^-1/2, g = exp(-exp(A_log) softplus(a + dt)).
+    Output: per-head RMS norm (weight shared by heads) * silu(gate) -> W_o.
+    """
+
+    def __init__(self, width, heads, kv_heads, dim, vdim, conv, eps, init):
+        super().__init__()
+        self.W, self.H, self.G, self.dk, self.dv = width, heads, kv_heads, dim, vdim
+        self.taps, self.eps = conv, eps
+        self.Cq = kv_heads * dim
+        self.Cv = heads * vdim
+        self.Cc = 2 * self.Cq + self.Cv
+        # fused rows: q | k | v | gate | beta | a
+        self.off_g = self.Cc
+        self.off_b = self.Cc + self.Cv
+        self.off_a = self.off_b + heads
+        self.w_in = init.mat(self.off_a + heads, width)
+        self.conv_w = init.vec((self.Cc, conv), -0.6, 0.9)
+        self.A_log = init.vec(heads, -4.0, -1.5)
+        self.dt_bias = init.vec(heads, -3.2, -2.8)
+        self.norm_w = init.vec(vdim, 0.7, 1.4)
+        self.w_o = init.mat(width, self.Cv)
+
+    def state_shapes(self):
+        return [(self.H, self.dk, self.dv), (self.taps - 1, self.Cc)]
+
+    def kv_shape(self):
+        return None
+
+    def load(self, get: Getter):
+        rows = [get("q"), get("k"), get("v"), get("g"), get("b"), get("a")]
+        _put(self.w_in, torch.cat(rows, 0))
+        _put(self.conv_w, torch.cat([get("q.conv"), get("k.conv"),
+                                     get("v.conv")], 0))
+        _put(self.A_log, get("A_log"))
+        _put(self.dt_bias, get("dt_bias"))
+        _put(self.norm_w, get("norm"))
+        _put(self.w_o, get("o"))
+
+    def forward(self, h, ctx: MixContext):
+        proj = F.linear(h, self.w_in)
+        S, conv_state = ctx.states
+        qkv = sops.causal_conv_silu(proj, self.Cc, self.conv_w, conv_state,
+                                    ctx.sb)
+        o = sops.gated_delta_rule(qkv, proj, self.off_b, self.off_a,
+                                  self.A_log, self.dt_bias, S, ctx.sb, self.H,
+                                  self.G, self.dv, self.dk ** -0.5)
+        y = sops.head_norm_gate(o, self.norm_w, 0, proj[:, self.off_g:],
+                                sops.GATE_SILU, self.eps, h.dtype)
+        return F.linear(y, self.w_o)
+
+
+class BiasedAttention(torch.nn.Module):
+    """Grouped-query softmax attention without rotation over the paged
+    cache. Options: query temperature 1 + coef ln(floor((p+1)/every) + 1),
+    RMS-normed values (cached normed), and a per-head distance penalty
+    r1 ln(1 + r2 (i - j)) subtracted from the scaled scores."""
+
+    def __init__(self, width, heads, kv_heads, dim, vdim, scale, eps, init,
+                 temp_coef=0.0, temp_every=1, value_norm=True,
+                 distance_bias=True):
+        super().__init__()
+        self.W, self.H, self.G, self.dk, self.dv = width, heads, kv_heads, dim, vdim
+        self.scale, self.eps = scale, eps
+        self.temp_coef, self.temp_every = temp_coef, temp_every
+        self.value_norm = value_norm
+        self.off_k = heads * dim
+        self.off_v = self.off_k + kv_heads * dim
+        self.w_in = init.mat(self.off_v + kv_heads * vdim, width)
+        self.r1 = init.vec(heads, 0.0, 2.0) if distance_bias else None
+        self.r2 = init.vec(heads, 0.1, 0.3) if distance_bias else None
+        self.w_o = init.mat(width, heads * vdim)
+
+    def state_shapes(self):
+        return []
+
+    def kv_shape(self):
+        return (self.G, self.dk, self.dv)
+
+    def load(self, get: Getter):
+        _put(self.w_in, torch.cat([get("q"), get("k"), get("v")], 0))
+        if self.r1 is not None:
+            _put(self.r1, get("r1"))
+            _put(self.r2, get("r2"))
+        _put(self.w_o, get("o"))
+
+    def forward(self, h, ctx: MixContext):
+        proj = F.linear(h, self.w_in)
+        sops.kv_append_norm(ctx.kcache, ctx.vcache, proj, self.off_k,
+                            self.off_v, ctx.slot_mapping, self.value_norm,
+                            self.eps)
+        y = sops.biased_attention(proj, 0, self.H, ctx.kcache, ctx.vcache,
+                                  ctx.positions, ctx.sb, self.r1, self.r2,
+                                  self.scale, self.temp_coef, self.temp_every)
+        return F.linear(y, self.w_o)
+
+
+class RWKVTimeMix(torch.nn.Module):
+    """RWKV-style time mixing: token-shift interpolations feed r, k, v, gate
+    and a low-rank data-dependent decay w = exp(-exp(W2 tanh(W1 x) + w0));
+    o = (S + diag(u) k v^T)^T r; S <- diag(w) S + k v^T.
+    Output: per-head RMS norm * weight * silu(gate) -> W_o."""
+
+    SHIFTS = ("r", "k", "v", "g", "w")
+
+    def __init__(self, width, heads, dim, eps, init, decay_rank=None):
+        super().__init__()
+        self.W, self.H, self.d, self.eps = width, heads, dim, eps
+        HD = heads * dim
+        rank = decay_rank or max(8, width // 16)
+        self.mu = init.vec((5, width), 0.0, 0.8)
+        # r, k, v, gate share a batched GEMM: [4, W, HD] (x @ w)
+        self.w_rkvg = torch.stack(
+            [init.mat(HD, width).t().contiguous() for _ in range(4)])
+        self.w1 = init.mat(rank, width)
+        self.w2 = init.mat(HD, rank, std=0.2)
+        self.w0 = init.vec(HD, -6.0, -1.0)
+        self.u = init.vec((heads, dim), -0.4, 1.4)
+        self.norm_w = init.vec(HD, 0.6, 1.4)
+        self.w_o = init.mat(width, HD)
+
+    def state_shapes(self):
+        return [(self.H, self.d, self.d), (self.W,)]
+
+    def kv_shape(self):
+        return None
+
+    def load(self, get: Getter):
+        _put(self.mu, torch.stack([get("mu." + s) for s in self.SHIFTS]))
+        _put(self.w_rkvg, torch.stack([get(s).t() for s in "rkvg"]))
+        if get("w1").shape != self.w1.shape:      # rank comes from the file
+            self.w1 = torch.empty_like(get("w1"), dtype=self.w1.dtype,
+                                       device=self.w1.device)
+            self.w2 = torch.empty_like(get("w2"), dtype=self.w2.dtype,
+                                       device=self.w2.device)
+        _put(self.w1, get("w1"))
+        _put(self.w2, get("w2"))
+        _put(self.w0, get("w0"))
+        _put(self.u, get("u"))
+        _put(self.norm_w, get("norm"))
+        _put(self.w_o, get("o"))
+
+    def forward(self, h, ctx: MixContext):
+        S, prev = ctx.states
+        mix = sops.token_shift_mix(h, self.mu, prev, ctx.sb)     # [5, T, W]
+        rkvg = torch.bmm(mix[:4], self.w_rkvg)                   # [4, T, HD]
+        wraw = F.linear(torch.tanh(F.linear(mix[4], self.w1)), self.w2)
+        o = sops.rwkv_time_mix(rkvg[0], rkvg[1], rkvg[2], wraw, self.w0,
+                               self.u, S, ctx.sb, self.H)
+        y = sops.head_norm_gate(o, self.norm_w, self.d, rkvg[3],
+                                sops.GATE_SILU, self.eps, h.dtype)
+        return F.linear(y, self.w_o)
+
+
+class MLSTMMixer(torch.nn.Module):
+    """mLSTM matrix memory with exponential gating, soft-capped gate
+    pre-activations and a running stabiliser that starts at 0.
+    Output: per-head RMS norm * weight * sigmoid(gate) -> W_o."""
+
+    def __init__(self, width, heads, dim, vdim, gate_cap, eps, init):
+        super().__init__()
+        self.W, self.H, self.dk, self.dv = width, heads, dim, vdim
+        self.cap, self.eps = gate_cap, eps
+        HK, HV = heads * dim, heads * vdim
+        # fused rows: q | k | v | gate | i | f
+        self.off_k, self.off_v, self.off_g = HK, 2 * HK, 2 * HK + HV
+        self.off_i = self.off_g + HV
+        self.off_f = self.off_i + heads
+        self.w_in = init.mat(self.off_f + heads, width)
+        self.i_bias = init.vec(heads, -1.0, 1.0)
+        self.f_bias = init.vec(heads, 1.0, 6.0)
+        self.norm_w = init.vec(HV, 0.6, 1.4)
+        self.w_o = init.mat(width, HV)
+
+    def state_shapes(self):
+        return [(self.H, self.dk, self.dv), (self.H, self.dk), (self.H,)]
+
+    def kv_shape(self):
+        return None
+
+    def load(self, get: Getter):
+        _put(self.w_in, torch.cat([get("q"), get("k"), get("v"), get("g"),
+                                   get("i"), get("f")], 0))
+        _put(self.i_bias, get("i.b"))
+        _put(self.f_bias, get("f.b"))
+        _put(self.norm_w, get("norm"))
+        _put(self.w_o, get("o"))
+
+    def forward(self, h, ctx: MixContext):
+        proj = F.linear(h, self.w_in)
+        S, n, m = ctx.states
+        o = sops.mlstm_memory(
+            proj, (0, self.off_k, self.off_v, self.off_i, self.off_f),
+            self.i_bias, self.f_bias, S, n, m, ctx.sb, self.H, self.dv,
+            self.dk ** -0.5, self.cap)
+        y = sops.head_norm_gate(o, self.norm_w, self.dv, proj[:, self.off_g:],
+                                sops.GATE_SIGMOID, self.eps, h.dtype)
+        return F.linear(y, self.w_o)
+
+
+class ParallelMixer(torch.nn.Module):
+    """Two mixers on the same input; the result is the mean of their
+    outputs, each RMS-normed over the width with its own weight."""
+
+    def __init__(self, width, left, right, eps, init):
+        super().__init__()
+        self.left, self.right, self.eps = left, right, eps
+        self.left_out = init.vec(width, 0.6, 1.3)
+        self.right_out = init.vec(width, 0.6, 1.3)
+
+    def state_shapes(self):
+        return self.left.state_shapes() + self.right.state_shapes()
+
+    def kv_shape(self):
+        return self.left.kv_shape() or self.right.kv_shape()
+
+    def load(self, get: Getter):
+        self.left.load(lambda n: get("left." + n))
+        self.right.load(lambda n: get("right." + n))
+        _put(self.left_out, get("left.out"))
+        _put(self.right_out, get("right.out"))
+
+    def forward(self, h, ctx: MixContext):
+        nl = len(self.left.state_shapes())
+        cl = MixContext(ctx.sb, ctx.positions, ctx.slot_mapping,
+                        ctx.states[:nl], ctx.kcache, ctx.vcache)
+        cr = MixContext(ctx.sb, ctx.positions, ctx.slot_mapping,
+                        ctx.states[nl:], ctx.kcache, ctx.vcache)
+        a = self.left.forward(h, cl)
+        b = self.right.forward(h, cr)
+        return sops.dual_rmsnorm_mean(a, b, self.left_out, self.right_out,
+                                      self.eps)
+
+
+class ClampedGLU(torch.nn.Module):
+    """Dense feed-forward: g = min(W_gate h, L); u = clamp(W_up h, -L, L);
+    W_down (g sigmoid(alpha g) (u + 1))."""
+
+    def __init__(self, width, ff, limit, init, alpha=1.702):
+        super().__init__()
+        self.limit, self.alpha = limit, alpha
+        self.w_gate_up = init.mat(2 * ff, width)
+        self.w_down = init.mat(width, ff)
+
+    def load(self, get: Getter):
+        _put(self.w_gate_up, torch.cat([get("gate"), get("up")], 0))
+        _put(self.w_down, get("down"))
+
+    def forward(self, h):
+        act = sops.clamped_glu(F.linear(h, self.w_gate_up), self.limit,
+                               self.alpha)
+        return F.linear(act, self.w_down)

@@ -14,6 +14,9 @@ def build_model(cfg: ModelConfig, device, dtype, tp=None, seed: int = 0):
     if cfg.arch == "mixtral":
         from .mixtral import MixtralForCausalLM
         return MixtralForCausalLM(cfg, device, dtype, tp, seed)
+    if cfg.arch == "bolatar":
+        from .bolatar import BolatarForCausalLM
+        return BolatarForCausalLM(cfg, device, dtype, tp, seed)
     raise ValueError(f"unknown arch {cfg.arch}")
 
 

@@ -1,0 +1,213 @@
+"""Sequence-mixer ops: recurrent matrix-state mixers (gated delta rule,
+RWKV-style time mixing, mLSTM), softmax attention with a distance bias over
+the paged cache, and their row-wise companions.
+
+GPU tensors go to the HIP kernels of dynamo_amd._hip_seq (required there -
+a missing extension raises); CPU tensors go to the plain torch versions in
+seq_ref. Both take the same arguments.
+
+The batch is the engine's flat run of token rows; `SeqBatch` says which rows
+belong to which sequence, where each sequence's portion starts in position
+space, and which state slot it owns. A decoded token is a portion of one.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Tuple
+
+import torch
+
+from . import seq_ref
+
+_mod = None
+
+
+def hip_seq():
+    global _mod
+    if _mod is None:
+        try:
+            from dynamo_amd import _hip_seq as m
+        except Exception as e:  # pragma: no cover
+            raise RuntimeError(
+                "dynamo_amd._hip_seq native extension is not available on a "
+                "GPU device path. Build it with `DYNAMO_AMD_EXTS=_hip_seq "
+                "python setup.py build_ext --inplace`. Original error: "
+                f"{e}") from e
+        _mod = m
+    return _mod
+
+
+@dataclass
+class SeqBatch:
+    tok_seq: torch.Tensor      # [T] int32: sequence index of each row
+    seq_start: torch.Tensor    # [B] int32: first row
+    seq_len: torch.Tensor      # [B] int32: rows this step (0 = padding)
+    seq_slot: torch.Tensor     # [B] int32: recurrent-state slot
+    seq_pos0: torch.Tensor     # [B] int32: position of the first row
+    page_table: Optional[torch.Tensor] = None   # [B, maxp] int32
+    # host copy [(start, len, slot, pos0)] for the CPU path
+    host: Optional[List[Tuple[int, int, int, int]]] = None
+
+    def spans(self):
+        if self.host is not None:
+            return self.host
+        return list(zip(self.seq_start.tolist(), self.seq_len.tolist(),
+                        self.seq_slot.tolist(), self.seq_pos0.tolist()))
+
+
+def _args(sb: SeqBatch):
+    return sb.seq_start, sb.seq_len, sb.seq_slot, sb.seq_pos0
+
+
+# -- row-wise ----------------------------------------------------------------
+def embed_scale_pos(ids, positions, embed, pos_table, scale: float):
+    """fp32 [T, W]: embed[id] * scale (+ pos_table[position])."""
+    if embed.is_cuda:
+        out = torch.empty(ids.shape[0], embed.shape[1], dtype=torch.float32,
+                          device=embed.device)
+        hip_seq().embed_scale_pos(out, ids, positions, embed, pos_table,
+                                  float(scale))
+        return out
+    return seq_ref.embed_scale_pos(ids, positions, embed, pos_table, scale)
+
+
+def add_scalar_rmsnorm(res, delta, g, eps: float, out_dtype):
+    """res (fp32, in place) += delta; returns res / rms(res) * g[0]."""
+    if res.is_cuda:
+        out = torch.empty(res.shape, dtype=out_dtype, device=res.device)
+        hip_seq().add_scalar_rmsnorm(out, res, delta, g, float(eps))
+        return out
+    return seq_ref.add_scalar_rmsnorm(res, delta, g, eps, out_dtype)
+
+
+def causal_conv_silu(x, C: int, w, conv_state, sb: SeqBatch):
+    """silu of a short causal convolution over the first C columns of x;
+    the slot's saved inputs continue earlier portions and are updated."""
+    if x.is_cuda:
+        out = torch.empty(x.shape[0], C, dtype=torch.float32, device=x.device)
+        hip_seq().causal_conv_silu(out, x, w, conv_state, sb.tok_seq,
+                                   *_args(sb))
+        return out
+    return seq_ref.causal_conv_silu(x, C, w, conv_state, sb)
+
+
+def token_shift_mix(h, mu, prev_state, sb: SeqBatch):
+    """[S, T, W]: h + (h_prev - h) * mu_s for each of the S rows of mu."""
+    if h.is_cuda:
+        out = torch.empty(mu.shape[0], *h.shape, dtype=h.dtype,
+                          device=h.device)
+        hip_seq().token_shift_mix(out, h, mu, prev_state, sb.tok_seq,
+                                  *_args(sb))
+        return out
+    return seq_ref.token_shift_mix(h, mu, prev_state, sb)
+
+
+GATE_NONE, GATE_SILU, GATE_SIGMOID = 0, 1, 2
+
+
+def head_norm_gate(o, w, w_stride: int, gate, gate_act: int, eps: float,
+                   out_dtype):
+    """o [T, H, dv] fp32 -> [T, H*dv]: per-head RMS norm, weight
+    w[h * w_stride + :], times act(gate[:, h*dv + :])."""
+    if o.is_cuda:
+        out = torch.empty(o.shape[0], o.shape[1] * o.shape[2], dtype=out_dtype,
+                          device=o.device)
+        hip_seq().head_norm_gate(out, o, w, w_stride, gate, gate_act,
+                                 float(eps))
+        return out
+    return seq_ref.head_norm_gate(o, w, w_stride, gate, gate_act, eps,
+                                  out_dtype)
+
+
+def clamped_glu(gate_up, limit: float, alpha: float):
+    """[T, 2F] (gate | up) -> min(g, L) * sigmoid(alpha g) * (clamp(u) + 1)."""
+    if gate_up.is_cuda:
+        out = torch.empty(gate_up.shape[0], gate_up.shape[1] // 2,
+                          dtype=gate_up.dtype, device=gate_up.device)
+        hip_seq().clamped_glu(out, gate_up, float(limit), float(alpha))
+        return out
+    return seq_ref.clamped_glu(gate_up, limit, alpha)
+
+
+def dual_rmsnorm_mean(a, b, wa, wb, eps: float):
+    if a.is_cuda:
+        out = torch.empty_like(a)
+        hip_seq().dual_rmsnorm_mean(out, a, b, wa, wb, float(eps))
+        return out
+    return seq_ref.dual_rmsnorm_mean(a, b, wa, wb, eps)
+
+
+def softcap_(x, cap: float):
+    if x.is_cuda:
+        hip_seq().softcap_(x, float(cap))
+        return x
+    return seq_ref.softcap_(x, cap)
+
+
+# -- recurrences ---------------------------------------------------------------
+def gated_delta_rule(qkv, proj, off_b: int, off_a: int, A_log, dt_bias, state,
+                     sb: SeqBatch, H: int, G: int, dv: int, qscale: float,
+                     unit_eps: float = 1e-6):
+    """qkv fp32 [T, 2*G*dk + H*dv]; gates read raw from proj. -> [T, H, dv]."""
+    if qkv.is_cuda:
+        out = torch.empty(qkv.shape[0], H, dv, dtype=torch.float32,
+                          device=qkv.device)
+        hip_seq().gated_delta_rule(out, qkv, proj, off_b, off_a, A_log,
+                                   dt_bias, state, *_args(sb), G,
+                                   float(qscale), float(unit_eps))
+        return out
+    return seq_ref.gated_delta_rule(qkv, proj, off_b, off_a, A_log, dt_bias,
+                                    state, sb, H, G, dv, qscale, unit_eps)
+
+
+def rwkv_time_mix(r, k, v, wraw, w0, u, state, sb: SeqBatch, H: int):
+    if r.is_cuda:
+        d = r.shape[1] // H
+        out = torch.empty(r.shape[0], H, d, dtype=torch.float32,
+                          device=r.device)
+        hip_seq().rwkv_time_mix(out, r, k, v, wraw, w0, u, state, *_args(sb))
+        return out
+    return seq_ref.rwkv_time_mix(r, k, v, wraw, w0, u, state, sb, H)
+
+
+def mlstm_memory(proj, offs, i_bias, f_bias, state_S, state_n, state_m,
+                 sb: SeqBatch, H: int, dv: int, qscale: float, cap: float,
+                 den_eps: float = 1e-6):
+    """offs = (q, k, v, i, f) column offsets into proj. -> [T, H, dv] fp32."""
+    if proj.is_cuda:
+        out = torch.empty(proj.shape[0], H, dv, dtype=torch.float32,
+                          device=proj.device)
+        hip_seq().mlstm_memory(out, proj, *offs, i_bias, f_bias, state_S,
+                               state_n, state_m, *_args(sb), float(qscale),
+                               float(cap), float(den_eps))
+        return out
+    return seq_ref.mlstm_memory(proj, offs, i_bias, f_bias, state_S, state_n,
+                                state_m, sb, H, dv, qscale, cap, den_eps)
+
+
+# -- attention -----------------------------------------------------------------
+def kv_append_norm(kcache, vcache, proj, off_k: int, off_v: int, slot_mapping,
+                   vnorm: bool, eps: float):
+    if proj.is_cuda:
+        hip_seq().kv_append_norm(kcache, vcache, proj, off_k, off_v,
+                                 slot_mapping, bool(vnorm), float(eps))
+    else:
+        seq_ref.kv_append_norm(kcache, vcache, proj, off_k, off_v,
+                               slot_mapping, vnorm, eps)
+
+
+def biased_attention(proj, off_q: int, H: int, kcache, vcache, positions,
+                     sb: SeqBatch, r1, r2, scale: float, temp_coef: float,
+                     temp_every: int):
+    """-> [T, H*dv] in proj's dtype."""
+    dv = vcache.shape[3]
+    if proj.is_cuda:
+        out = torch.empty(proj.shape[0], H, dv, dtype=proj.dtype,
+                          device=proj.device)
+        hip_seq().biased_attention(out, proj, off_q, kcache, vcache,
+                                   sb.page_table, sb.tok_seq, positions,
+                                   sb.seq_len, r1, r2, float(scale),
+                                   float(temp_coef), int(temp_every))
+        return out.view(proj.shape[0], H * dv)
+    return seq_ref.biased_attention(proj, off_q, H, kcache, vcache, positions,
+                                    sb, r1, r2, scale, temp_coef, temp_every)

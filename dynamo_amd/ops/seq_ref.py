@@ -1,0 +1,231 @@
+"""Plain torch versions of the sequence-mixer ops (the CPU path).
+
+Same arguments and state layout as the HIP kernels: fp32 state tensors
+indexed by slot, a portion that starts at position 0 ignores what its slot
+holds. Token loops are explicit; this path is for CPU engines and tests.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def embed_scale_pos(ids, positions, embed, pos_table, scale):
+    x = embed[ids.long()].float() * scale
+    if pos_table is not None:
+        x = x + pos_table[positions.long()].float()
+    return x
+
+
+def add_scalar_rmsnorm(res, delta, g, eps, out_dtype):
+    if delta is not None:
+        res.add_(delta.float())
+    inv = torch.rsqrt(res.pow(2).mean(-1, keepdim=True) + eps)
+    return (res * inv * g.float().reshape(())).to(out_dtype)
+
+
+def causal_conv_silu(x, C, w, conv_state, sb):
+    taps = w.shape[1]
+    K = taps - 1
+    xin = x[:, :C].float()
+    out = torch.empty(x.shape[0], C, dtype=torch.float32)
+    for start, n, slot, pos0 in sb.spans():
+        if n == 0:
+            continue
+        hist = (conv_state[slot].clone() if pos0 > 0
+                else torch.zeros(K, C, dtype=torch.float32))
+        if 0 < pos0 < K:
+            hist[:K - pos0] = 0
+        full = torch.cat([hist, xin[start:start + n]], 0)      # [K + n, C]
+        acc = torch.zeros(n, C, dtype=torch.float32)
+        for j in range(taps):
+            acc += full[j:j + n] * w[:, j]
+        out[start:start + n] = F.silu(acc)
+        if K:
+            conv_state[slot] = full[-K:]
+    return out
+
+
+def token_shift_mix(h, mu, prev_state, sb):
+    hf = h.float()
+    prev = torch.zeros_like(hf)
+    for start, n, slot, pos0 in sb.spans():
+        if n == 0:
+            continue
+        if pos0 > 0:
+            prev[start] = prev_state[slot]
+        prev[start + 1:start + n] = hf[start:start + n - 1]
+        prev_state[slot] = hf[start + n - 1]
+    return (hf.unsqueeze(0) + (prev - hf).unsqueeze(0) *
+            mu.float().unsqueeze(1)).to(h.dtype)
+
+
+def head_norm_gate(o, w, w_stride, gate, gate_act, eps, out_dtype):
+    T, H, dv = o.shape
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+    wh = torch.stack([w[h * w_stride:h * w_stride + dv] for h in range(H)])
+    y = y * wh
+    if gate_act:
+        g = gate[:, :H * dv].float().view(T, H, dv)
+        y = y * (F.silu(g) if gate_act == 1 else torch.sigmoid(g))
+    return y.reshape(T, H * dv).to(out_dtype)
+
+
+def clamped_glu(gate_up, limit, alpha):
+    Fd = gate_up.shape[1] // 2
+    g = gate_up[:, :Fd].float().clamp(max=limit)
+    u = gate_up[:, Fd:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1)).to(gate_up.dtype)
+
+
+def dual_rmsnorm_mean(a, b, wa, wb, eps):
+    def n(x, w):
+        x = x.float()
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w
+    return (0.5 * (n(a, wa) + n(b, wb))).to(a.dtype)
+
+
+def softcap_(x, cap):
+    return x.copy_(cap * torch.tanh(x / cap))
+
+
+def gated_delta_rule(qkv, proj, off_b, off_a, A_log, dt_bias, state, sb, H, G,
+                     dv, qscale, unit_eps):
+    T = qkv.shape[0]
+    dk = state.shape[2]
+    Cq = G * dk
+    q = qkv[:, :Cq].view(T, G, dk)
+    k = qkv[:, Cq:2 * Cq].view(T, G, dk)
+    v = qkv[:, 2 * Cq:].view(T, H, dv)
+    q = q / torch.sqrt(q.pow(2).sum(-1, keepdim=True) + unit_eps) * qscale
+    k = k / torch.sqrt(k.pow(2).sum(-1, keepdim=True) + unit_eps)
+    beta = torch.sigmoid(proj[:, off_b:off_b + H].float())
+    g = torch.exp(-torch.exp(A_log) *
+                  F.softplus(proj[:, off_a:off_a + H].float() + dt_bias))
+    rep = H // G
+    out = torch.empty(T, H, dv, dtype=torch.float32)
+    for start, n, slot, pos0 in sb.spans():
+        if n == 0:
+            continue
+        S = state[slot].clone() if pos0 > 0 else torch.zeros_like(state[slot])
+        for t in range(start, start + n):
+            kt = k[t].repeat_interleave(rep, 0)            # [H, dk]
+            qt = q[t].repeat_interleave(rep, 0)
+            S = S * g[t].view(H, 1, 1)
+            u = beta[t].view(H, 1) * (v[t] - torch.einsum("hkv,hk->hv", S, kt))
+            S = S + kt.unsqueeze(2) * u.unsqueeze(1)
+            out[t] = torch.einsum("hkv,hk->hv", S, qt)
+        state[slot] = S
+    return out
+
+
+def rwkv_time_mix(r, k, v, wraw, w0, u, state, sb, H):
+    T = r.shape[0]
+    d = r.shape[1] // H
+    r, k, v = (x.float().view(T, H, d) for x in (r, k, v))
+    w = torch.exp(-torch.exp(wraw.float() + w0)).view(T, H, d)
+    uu = u.view(H, d)
+    out = torch.empty(T, H, d, dtype=torch.float32)
+    for start, n, slot, pos0 in sb.spans():
+        if n == 0:
+            continue
+        S = state[slot].clone() if pos0 > 0 else torch.zeros_like(state[slot])
+        for t in range(start, start + n):
+            kv = k[t].unsqueeze(2) * v[t].unsqueeze(1)       # [H, d, d]
+            out[t] = torch.einsum("hkv,hk->hv", S + uu.unsqueeze(2) * kv, r[t])
+            S = w[t].unsqueeze(2) * S + kv
+        state[slot] = S
+    return out
+
+
+def mlstm_memory(proj, offs, i_bias, f_bias, state_S, state_n, state_m, sb, H,
+                 dv, qscale, cap, den_eps):
+    T = proj.shape[0]
+    dk = state_S.shape[2]
+    oq, ok, ov, oi, of = offs
+    p = proj.float()
+    q = p[:, oq:oq + H * dk].view(T, H, dk) * qscale
+    k = p[:, ok:ok + H * dk].view(T, H, dk)
+    v = p[:, ov:ov + H * dv].view(T, H, dv)
+    ig = cap * torch.tanh((p[:, oi:oi + H] + i_bias) / cap)
+    fg = F.logsigmoid(cap * torch.tanh((p[:, of:of + H] + f_bias) / cap))
+    out = torch.empty(T, H, dv, dtype=torch.float32)
+    for start, n, slot, pos0 in sb.spans():
+        if n == 0:
+            continue
+        if pos0 > 0:
+            S, nn, m = (state_S[slot].clone(), state_n[slot].clone(),
+                        state_m[slot].clone())
+        else:
+            S, nn, m = (torch.zeros_like(state_S[slot]),
+                        torch.zeros_like(state_n[slot]),
+                        torch.zeros_like(state_m[slot]))
+        for t in range(start, start + n):
+            mn = torch.maximum(fg[t] + m, ig[t])
+            a, b = torch.exp(fg[t] + m - mn), torch.exp(ig[t] - mn)
+            m = mn
+            S = a.view(H, 1, 1) * S + b.view(H, 1, 1) * (
+                k[t].unsqueeze(2) * v[t].unsqueeze(1))
+            nn = a.view(H, 1) * nn + b.view(H, 1) * k[t]
+            num = torch.einsum("hkv,hk->hv", S, q[t])
+            nq = (nn * q[t]).sum(-1)
+            den = torch.maximum(nq.abs(), torch.exp(-m)) + den_eps
+            out[t] = num / den.view(H, 1)
+        state_S[slot], state_n[slot], state_m[slot] = S, nn, m
+    return out
+
+
+def kv_append_norm(kcache, vcache, proj, off_k, off_v, slot_mapping, vnorm,
+                   eps):
+    P, G, ps, dk = kcache.shape
+    dv = vcache.shape[3]
+    T = proj.shape[0]
+    k = proj[:, off_k:off_k + G * dk].view(T, G, dk)
+    v = proj[:, off_v:off_v + G * dv].float().view(T, G, dv)
+    if vnorm:
+        v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    v = v.to(vcache.dtype)
+    for t, slot in enumerate(slot_mapping.tolist()):
+        if slot < 0:
+            continue
+        kcache[slot // ps, :, slot % ps] = k[t]
+        vcache[slot // ps, :, slot % ps] = v[t]
+
+
+def biased_attention(proj, off_q, H, kcache, vcache, positions, sb, r1, r2,
+                     scale, temp_coef, temp_every):
+    P, G, ps, dk = kcache.shape
+    dv = vcache.shape[3]
+    T = proj.shape[0]
+    q = proj[:, off_q:off_q + H * dk].float().view(T, H, dk)
+    out = torch.zeros(T, H, dv, dtype=torch.float32)
+    pos = positions.tolist()
+    rep = H // G
+    for si, (start, n, slot, pos0) in enumerate(sb.spans()):
+        if n == 0:
+            continue
+        pages = sb.page_table[si].long()
+        ctx = pos0 + n
+        npg = (ctx + ps - 1) // ps
+        # [G, ctx, d] gathered from the pages
+        kk = kcache[pages[:npg]].float().permute(1, 0, 2, 3).reshape(
+            G, npg * ps, dk)[:, :ctx]
+        vv = vcache[pages[:npg]].float().permute(1, 0, 2, 3).reshape(
+            G, npg * ps, dv)[:, :ctx]
+        kk = kk.repeat_interleave(rep, 0)
+        vv = vv.repeat_interleave(rep, 0)
+        for t in range(start, start + n):
+            i = pos[t]
+            temp = 1.0
+            if temp_coef != 0.0:
+                temp += temp_coef * math.log((i + 1) // temp_every + 1)
+            s = torch.einsum("hd,hjd->hj", q[t] * (temp * scale),
+                             kk[:, :i + 1])
+            if r1 is not None:
+                dist = (i - torch.arange(i + 1)).float()
+                s = s - r1.view(H, 1) * torch.log1p(r2.view(H, 1) * dist)
+            out[t] = torch.einsum("hj,hjd->hd", torch.softmax(s, -1),
+                                  vv[:, :i + 1])
+    return out.to(proj.dtype).view(T, H * dv)

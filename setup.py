@@ -32,13 +32,34 @@ hip_sources = [
     )
 ]
 
+SEQ = os.path.join(CSRC, "seqmix")
+seq_sources = [
+    os.path.join(SEQ, f)
+    for f in ("seq_bindings.cpp", "seq_elementwise.hip", "seq_recurrence.hip",
+              "seq_attention.hip")
+]
+
+# hipcc emits packed-fp32 VALU ops from plain float code unless told not to
+HIPCC_FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
 ext_modules = [
     CUDAExtension(
         name="dynamo_amd._hip",
         sources=hip_sources,
         extra_compile_args={
             "cxx": ["-O3", "-std=c++17"],
-            "nvcc": ["-O3", "-std=c++17", "--offload-arch=gfx950"],
+            "nvcc": HIPCC_FLAGS,
+        },
+    ),
+    # recurrent / biased-attention mixers: a separate module so a model that
+    # needs only these builds without the MFMA attention kernels
+    CUDAExtension(
+        name="dynamo_amd._hip_seq",
+        sources=seq_sources,
+        extra_compile_args={
+            "cxx": ["-O3", "-std=c++17"],
+            "nvcc": HIPCC_FLAGS,
         },
     ),
     CppExtension(
@@ -47,6 +68,12 @@ ext_modules = [
         extra_compile_args=["-O3", "-std=c++17"],
     ),
 ]
+
+# DYNAMO_AMD_EXTS=_core,_hip_seq builds a subset (first-use builds of one
+# model family); unset builds everything
+_only = [e for e in os.environ.get("DYNAMO_AMD_EXTS", "").split(",") if e]
+if _only:
+    ext_modules = [e for e in ext_modules if e.name.split(".")[-1] in _only]
 
 setup(
     name="dynamo_amd",
