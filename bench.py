@@ -25,6 +25,7 @@ import argparse
 import json
 import os
 import random
+import sys
 import statistics
 import time
 
@@ -52,6 +53,12 @@ def parse_args():
                    help="V-page layout: auto = d-major on GPU when supported")
     p.add_argument("--device", default=None, help="cpu for gloo testing")
     p.add_argument("--max-batched-tokens", type=int, default=0)
+    p.add_argument("--mixer-compare", action="store_true",
+                   help="instead of the flagship workload: prefill/decode "
+                        "throughput of the layer-list (Bolatar) design "
+                        "beside Llama at equal sizes (1 GPU)")
+    p.add_argument("--mixer-sizes", default="small,medium",
+                   help="comma list of benchmarks/mixer_compare.py SIZES")
     p.add_argument("--moe-ep", action="store_true",
                    help="expert parallelism for MoE models (auto for N>1)")
     return p.parse_args()
@@ -450,6 +457,12 @@ def main():
         torch.cuda.set_device(local_rank)
         from dynamo_amd.utils import enable_tunableop
         enable_tunableop(tuning=False)
+    if args.mixer_compare:
+        sys.path.insert(0, os.path.join(os.path.dirname(
+            os.path.abspath(__file__)), "benchmarks"))
+        import mixer_compare
+        mixer_compare.run(args.mixer_sizes.split(","), device)
+        return
     if world > 1:
         dist.init_process_group("nccl" if device.startswith("cuda") else "gloo")
 

@@ -1,0 +1,139 @@
+"""Prefill and decode throughput of the layer-list (Bolatar) design beside
+the dense-attention Llama layout at equal width, depth, feed-forward size
+and vocabulary, random weights, one GPU, through the engine's own
+add_request/step loop (chunked prefill, then hipGraph decode).
+
+    python bench.py --mixer-compare [--mixer-sizes small,medium]
+
+Prints one JSON line: per size and model, prefill tokens/s (B prompts of
+ISL tokens until every request has its first token) and decode tokens/s
+(the following steps, all requests decoding).
+"""
+from __future__ import annotations
+
+import json
+import time
+
+import torch
+
+SIZES = {
+    # width, layers, ff, prompts, isl, decode batch, decode steps
+    "small": dict(width=1024, layers=4, ff=4096, prompts=4, isl=1024,
+                  conc=32, steps=64),
+    "medium": dict(width=2048, layers=8, ff=8192, prompts=4, isl=2048,
+                   conc=32, steps=64),
+    "wide": dict(width=4096, layers=4, ff=14336, prompts=2, isl=2048,
+                 conc=64, steps=48),
+}
+VOCAB = 32000
+
+
+def bolatar_config(width, layers, ff):
+    from dynamo_amd.engine.config import ModelConfig
+    hd = 128
+    H = width // hd
+    mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+    delta = {"type": "delta", "mlp": mlp,
+             "mixer": {"heads": H, "kv_heads": max(1, H // 2), "dim": hd,
+                       "vdim": hd, "conv": 4}}
+    par = {"type": "parallel", "mlp": mlp,
+           "mixer": {"left": {"heads": H, "kv_heads": max(1, H // 4),
+                              "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                              "q_temp": {"coef": 0.1, "every": 1024}},
+                     "right": {"heads": width // 64, "dim": 64}}}
+    mlstm = {"type": "mlstm", "mlp": mlp,
+             "mixer": {"heads": max(1, H // 2), "dim": hd, "vdim": 2 * hd,
+                       "gate_cap": 15.0}}
+    pattern = [delta, par, mlstm, delta]
+    specs = [pattern[i % 4] for i in range(layers)]
+    return ModelConfig(name=f"bolatar-w{width}", arch="bolatar",
+                       hidden_size=width, vocab_size=VOCAB, max_position=8192,
+                       num_layers=layers, rms_eps=1e-6, learned_pos_emb=True,
+                       layer_specs=specs, embed_scale=1.0, logit_softcap=30.0,
+                       intermediate_size=0, num_q_heads=1, num_kv_heads=1,
+                       head_dim=1)
+
+
+def llama_config(width, layers, ff):
+    from dynamo_amd.engine.config import ModelConfig
+    H = width // 128
+    return ModelConfig(name=f"llama-w{width}", arch="llama", hidden_size=width,
+                       intermediate_size=ff, num_layers=layers, num_q_heads=H,
+                       num_kv_heads=max(1, H // 4), head_dim=128,
+                       vocab_size=VOCAB, max_position=8192, rope_theta=1e4)
+
+
+def measure(mc, s, device):
+    from dynamo_amd.engine import EngineConfig, LLMEngine, SamplingParams
+    n = max(s["prompts"], s["conc"])
+    cfg = EngineConfig(model=mc, device=device, dtype="bfloat16",
+                       page_size=64, max_num_seqs=n,
+                       max_batched_tokens=s["prompts"] * s["isl"],
+                       max_model_len=s["isl"] + s["steps"] + 128,
+                       kv_pool_pages=n * ((s["isl"] + s["steps"]) // 64 + 3),
+                       enable_prefix_caching=False, kv_events=False)
+    eng = LLMEngine(cfg, seed=0)
+    g = torch.Generator().manual_seed(0)
+
+    def prompts(k, tag):
+        for i in range(k):
+            toks = torch.randint(0, mc.vocab_size, (s["isl"],), generator=g)
+            eng.add_request(f"{tag}{i}", toks.tolist(),
+                            SamplingParams(max_tokens=s["steps"] + 8,
+                                           ignore_eos=True))
+
+    def drain_until(pred):
+        while eng.has_work() and not pred():
+            eng.step()
+        torch.cuda.synchronize()
+
+    def first_tokens():
+        return all(r.output_tokens for r in eng.requests.values())
+
+    # warm-up: one prompt through prefill and a few decode steps
+    prompts(1, "w")
+    drain_until(first_tokens)
+    for _ in range(3):
+        eng.step()
+    for rid in list(eng.requests):
+        eng.abort(rid)
+    torch.cuda.synchronize()
+
+    prompts(s["prompts"], "p")
+    t0 = time.perf_counter()
+    drain_until(first_tokens)
+    prefill_s = time.perf_counter() - t0
+    # fill up to the decode batch (untimed), then time pure decode steps
+    prompts(s["conc"] - s["prompts"], "d")
+    drain_until(first_tokens)
+    for _ in range(4):           # graph capture for this batch size
+        eng.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    done = 0
+    for _ in range(s["steps"] - 8):
+        done += len(eng.step())
+    torch.cuda.synchronize()
+    decode_s = time.perf_counter() - t0
+    out = {"prefill_tok_s": round(s["prompts"] * s["isl"] / prefill_s, 1),
+           "decode_tok_s": round(done / decode_s, 1),
+           "decode_ms_per_step": round(1000 * decode_s / (s["steps"] - 8), 3)}
+    del eng
+    torch.cuda.empty_cache()
+    return out
+
+
+def run(sizes, device="cuda:0"):
+    res = {}
+    for name in sizes:
+        s = SIZES[name]
+        args = (s["width"], s["layers"], s["ff"])
+        res[name] = {
+            "shape": {k: s[k] for k in ("width", "layers", "ff", "prompts",
+                                        "isl", "conc")},
+            "bolatar": measure(bolatar_config(*args), s, device),
+            "llama": measure(llama_config(*args), s, device)}
+        print(f"# {name}: {json.dumps(res[name])}", flush=True)
+    print(json.dumps({"metric": "mixer_compare", "dtype": "bf16",
+                      "data": "synthetic", "sizes": res}), flush=True)
+    return res

@@ -351,6 +351,8 @@ class LLMEngine:
             n = len(tokens)
             if n == 0:
                 continue
+            if min(tokens) < 0 or max(tokens) >= self.cfg.model.vocab_size:
+                raise ValueError(f"{req_id}: token id outside the vocabulary")
             req.prompt_tokens.extend(int(t) for t in tokens)
             if req.total_len > self.cfg.max_model_len:
                 raise ValueError(f"{req_id} exceeds max_model_len")

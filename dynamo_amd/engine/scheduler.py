@@ -161,6 +161,9 @@ class Scheduler:
             if victim is exclude:
                 continue
             self.running.pop(i)
+            # the victim may already hold a place in this step's batch
+            out.decodes = [x for x in out.decodes if x.req is not victim]
+            out.prefills = [x for x in out.prefills if x.req is not victim]
             victim.kv.release()
             victim.kv = None
             self._release_state(victim)

@@ -86,10 +86,9 @@ def biased_attention(h, W, p, m, eps):
         for hh in range(H):
             kv = hh // (H // G)
             r1, r2 = W[p + "r1"][hh], W[p + "r2"][hh]
-            s = torch.empty(i + 1, dtype=F64)
-            for j in range(i + 1):
-                s[j] = (q[i, hh] * temp) @ k[j, kv] * m["scale"] \
-                    - r1 * torch.log(1 + r2 * (i - j))
+            dist = (i - torch.arange(i + 1)).to(F64)
+            s = (k[:i + 1, kv] @ (q[i, hh] * temp)) * m["scale"] \
+                - r1 * torch.log(1 + r2 * dist)
             a = torch.softmax(s, 0)
             out[i, hh] = a @ v[:i + 1, kv]
     return out.reshape(T, H * dv) @ W[p + "o"].T
