@@ -1,9 +1,9 @@
 // Softmax attention over the paged cache with a logarithmic distance bias
 // and a position-dependent query temperature, for head sizes the MFMA
 // flash kernels do not cover (any dk, dv up to 64 * EVMAX) and for fp32
-// caches. One wave per (token row, query head): lanes own keys for the
-// score pass and value channels for the weighted sum. Scores, softmax and
-// the accumulator are fp32.
+// caches. One workgroup per (token row, group of query heads sharing a kv
+// head); see biased_attention_kernel. Scores, softmax and the accumulator
+// are fp32.
 //
 //   score(i, j) = temp(i) * scale * (q_i . k_j) - r1_h * log1p(r2_h * (i - j))
 //   temp(i)     = 1 + coef * ln(floor((i + 1) / every) + 1)
@@ -47,8 +47,35 @@ __global__ void kv_append_norm_kernel(
   for (int i = lane; i < dv; i += 64) vd[i] = from_f<T>(to_f(vrow[i]) * inv);
 }
 
-template <typename T>
-__global__ void biased_attention_kernel(
+// 16-byte vector of activations
+template <typename T> struct Vec16;
+template <> struct Vec16<float> {
+  static constexpr int N = 4;
+  float4 v;
+  DEVINL float get(int i) const { return (&v.x)[i]; }
+};
+template <> struct Vec16<bf16_t> {
+  static constexpr int N = 8;
+  uint4 v;
+  DEVINL float get(int i) const {
+    const uint32_t w = (&v.x)[i >> 1];
+    union { float f; uint32_t u; } c;
+    c.u = (i & 1) ? (w & 0xffff0000u) : (w << 16);
+    return c.f;
+  }
+};
+
+// One workgroup (4 waves) per (token row, group of GS query heads that
+// share a kv head). The waves take 64-key chunks in turn and are merged
+// through LDS at the end, so a decoded token with a long context still
+// spreads over 4 waves. Within a chunk, 4 adjacent lanes share a key:
+// each reads every 4th 16-byte piece of the key row (a quad covers 64
+// contiguous bytes) and the quad adds its partial dots, 16 keys a pass, 4
+// passes a chunk; no transposed staging is needed. For the weighted sum
+// lanes own value channels and read value rows as they lie in the page.
+// VEC is off when a key row is not a whole number of 16-byte pieces.
+template <typename T, int GS, bool VEC>
+__global__ __launch_bounds__(256) void biased_attention_kernel(
     T* __restrict__ out,  // [T, H, dv]
     const T* __restrict__ proj, int proj_stride, int off_q,
     const T* __restrict__ kcache, const T* __restrict__ vcache,
@@ -57,65 +84,193 @@ __global__ void biased_attention_kernel(
     const int* __restrict__ seq_len, const float* __restrict__ r1,
     const float* __restrict__ r2, int H, int G, int dk, int dv, int ps,
     float scale, float temp_coef, int temp_every, int has_bias) {
-  extern __shared__ float qs[];  // [dk] scaled query
-  const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+  extern __shared__ float lds[];  // q [GS][dk]; merge [4][GS][2 + dv]
+  constexpr int VN = Vec16<T>::N;
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int s = tok_seq[t];
   if (seq_len[s] == 0) return;  // padding row
+  const int h0 = blockIdx.y * GS;  // first query head of this group
+  const int g = h0 / (H / G);
   const int pos = positions[t];
-  const int g = hh / (H / G);
   float temp = 1.f;
   if (temp_coef != 0.f)
     temp += temp_coef * logf((float)((pos + 1) / temp_every) + 1.f);
   const float qmul = temp * scale;
-  const T* q = proj + (int64_t)t * proj_stride + off_q + hh * dk;
-  for (int i = lane; i < dk; i += 64) qs[i] = to_f(q[i]) * qmul;
+  float* qs = lds;
+  float* mg = lds + GS * dk;
+  for (int i = threadIdx.x; i < GS * dk; i += 256)
+    qs[i] = to_f(proj[(int64_t)t * proj_stride + off_q + h0 * dk + i]) * qmul;
   __syncthreads();
   const int* table = page_table + (int64_t)s * table_stride;
-  const float b1 = has_bias ? r1[hh] : 0.f;
-  const float b2 = has_bias ? r2[hh] : 0.f;
+  float b1[GS], b2[GS];
+#pragma unroll
+  for (int a = 0; a < GS; a++) {
+    b1[a] = has_bias ? r1[h0 + a] : 0.f;
+    b2[a] = has_bias ? r2[h0 + a] : 0.f;
+  }
+  const int quad = lane >> 2, qq = lane & 3;
+  const int nvec = dk / VN;  // used when VEC
 
-  float m = -INFINITY, l = 0.f;
-  float acc[EVMAX];
+  float m[GS], l[GS], acc[GS][EVMAX];
 #pragma unroll
-  for (int e = 0; e < EVMAX; e++) acc[e] = 0.f;
+  for (int a = 0; a < GS; a++) {
+    m[a] = -INFINITY;
+    l[a] = 0.f;
+#pragma unroll
+    for (int e = 0; e < EVMAX; e++) acc[a][e] = 0.f;
+  }
   const int ctx = pos + 1;
-  for (int j0 = 0; j0 < ctx; j0 += 64) {
-    const int j = j0 + lane;
-    float sc = -INFINITY;
-    if (j < ctx) {
-      const int64_t page = table[j / ps];
-      const T* k = kcache + ((page * G + g) * ps + (j % ps)) * dk;
-      float d = 0.f;
-      for (int i = 0; i < dk; i++) d += qs[i] * to_f(k[i]);
-      sc = d;
-      if (has_bias) sc -= b1 * log1pf(b2 * (float)(pos - j));
+  const int nchunks = (ctx + 63) >> 6;
+  for (int c = wave; c < nchunks; c += 4) {
+    const int j0 = c << 6;
+    // ---- scores: pass p covers keys j0 + 16 p + quad ----
+    float sc[4][GS];
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      const int j = j0 + 16 * p + quad;
+      float d[GS];
+#pragma unroll
+      for (int a = 0; a < GS; a++) d[a] = 0.f;
+      if (j < ctx) {
+        const int64_t page = table[j / ps];
+        const T* k = kcache + ((page * G + g) * ps + (j % ps)) * dk;
+        if (VEC) {
+          for (int v = qq; v < nvec; v += 4) {
+            Vec16<T> kv;
+            kv.v = *reinterpret_cast<const decltype(kv.v)*>(k + v * VN);
+#pragma unroll
+            for (int i = 0; i < VN; i++) {
+              const float kf = kv.get(i);
+#pragma unroll
+              for (int a = 0; a < GS; a++) d[a] += qs[a * dk + v * VN + i] * kf;
+            }
+          }
+        } else {
+          for (int i = qq; i < dk; i += 4) {
+            const float kf = to_f(k[i]);
+#pragma unroll
+            for (int a = 0; a < GS; a++) d[a] += qs[a * dk + i] * kf;
+          }
+        }
+      }
+#pragma unroll
+      for (int a = 0; a < GS; a++) {
+        float x = d[a];
+        x += __shfl_xor(x, 1, 64);
+        x += __shfl_xor(x, 2, 64);
+        if (j < ctx) {
+          if (has_bias) x -= b1[a] * log1pf(b2[a] * (float)(pos - j));
+        } else {
+          x = -INFINITY;
+        }
+        sc[p][a] = x;
+      }
     }
-    const float mn = fmaxf(m, wave_max(sc));
-    const float corr = expf(m - mn);  // 0 on the first chunk (m = -inf)
-    const float p = (j < ctx) ? expf(sc - mn) : 0.f;
-    l = l * corr + wave_sum(p);
-    m = mn;
+    // ---- online softmax (every lane of a quad holds the same score) ----
+    float pr[4][GS];
 #pragma unroll
-    for (int e = 0; e < EVMAX; e++) acc[e] *= corr;
-    const int n = min(64, ctx - j0);
-    for (int jj = 0; jj < n; jj++) {
-      const float pj = __shfl(p, jj, 64);
-      const int jk = j0 + jj;
-      const int64_t page = table[jk / ps];
-      const T* v = vcache + ((page * G + g) * ps + (jk % ps)) * dv;
+    for (int a = 0; a < GS; a++) {
+      float mx = fmaxf(fmaxf(sc[0][a], sc[1][a]), fmaxf(sc[2][a], sc[3][a]));
+      mx = fmaxf(m[a], wave_max(mx));
+      const float corr = expf(m[a] - mx);
+      float sum = 0.f;
 #pragma unroll
-      for (int e = 0; e < EVMAX; e++) {
-        const int c = lane + 64 * e;
-        if (c < dv) acc[e] += pj * to_f(v[c]);
+      for (int p = 0; p < 4; p++) {
+        pr[p][a] = expf(sc[p][a] - mx);  // 0 for masked keys
+        sum += pr[p][a];
+      }
+      l[a] = l[a] * corr + 0.25f * wave_sum(sum);  // 4 lanes per key
+      m[a] = mx;
+#pragma unroll
+      for (int e = 0; e < EVMAX; e++) acc[a][e] *= corr;
+    }
+    // ---- weighted sum of values: lanes own channels ----
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      const int nk = min(16, ctx - (j0 + 16 * p));
+      for (int kk = 0; kk < nk; kk++) {
+        const int j = j0 + 16 * p + kk;
+        const int64_t page = table[j / ps];
+        const T* v = vcache + ((page * G + g) * ps + (j % ps)) * dv;
+        float w[GS];
+#pragma unroll
+        for (int a = 0; a < GS; a++) w[a] = __shfl(pr[p][a], kk << 2, 64);
+#pragma unroll
+        for (int e = 0; e < EVMAX; e++) {
+          const int ch = lane + 64 * e;
+          if (ch < dv) {
+            const float vf = to_f(v[ch]);
+#pragma unroll
+            for (int a = 0; a < GS; a++) acc[a][e] += w[a] * vf;
+          }
+        }
       }
     }
   }
-  const float inv = 1.f / l;
+  // ---- merge the 4 waves ----
+  const int MS = 2 + dv;  // floats per (wave, head) record
 #pragma unroll
-  for (int e = 0; e < EVMAX; e++) {
-    const int c = lane + 64 * e;
-    if (c < dv) out[((int64_t)t * H + hh) * dv + c] = from_f<T>(acc[e] * inv);
+  for (int a = 0; a < GS; a++) {
+    float* rec = mg + (wave * GS + a) * MS;
+    if (lane == 0) {
+      rec[0] = m[a];
+      rec[1] = l[a];
+    }
+#pragma unroll
+    for (int e = 0; e < EVMAX; e++) {
+      const int ch = lane + 64 * e;
+      if (ch < dv) rec[2 + ch] = acc[a][e];
+    }
   }
+  __syncthreads();
+  for (int a = wave; a < GS; a += 4) {  // wave a finishes head a
+    float mx = -INFINITY;
+    for (int w = 0; w < 4; w++) mx = fmaxf(mx, mg[(w * GS + a) * MS]);
+    float lt = 0.f, f[4];
+    for (int w = 0; w < 4; w++) {
+      const float mw = mg[(w * GS + a) * MS];
+      f[w] = (mw == -INFINITY) ? 0.f : expf(mw - mx);
+      lt += f[w] * mg[(w * GS + a) * MS + 1];
+    }
+    const float inv = 1.f / lt;
+    for (int ch = lane; ch < dv; ch += 64) {
+      float o = 0.f;
+      for (int w = 0; w < 4; w++) o += f[w] * mg[(w * GS + a) * MS + 2 + ch];
+      out[((int64_t)t * H + h0 + a) * dv + ch] = from_f<T>(o * inv);
+    }
+  }
+}
+
+template <typename T>
+void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
+                      torch::Tensor& kcache, torch::Tensor& vcache,
+                      torch::Tensor& page_table, torch::Tensor& tok_seq,
+                      torch::Tensor& positions, torch::Tensor& seq_len,
+                      c10::optional<torch::Tensor>& r1,
+                      c10::optional<torch::Tensor>& r2, double scale,
+                      double temp_coef, int64_t temp_every) {
+  const int T_ = out.size(0), H = out.size(1), dv = out.size(2);
+  const int G = kcache.size(1), ps = kcache.size(2), dk = kcache.size(3);
+  const int gsz = H / G;
+  const int GS = gsz % 4 == 0 ? 4 : (gsz % 2 == 0 ? 2 : 1);
+  const size_t lds = (size_t)(GS * dk + 4 * GS * (2 + dv)) * sizeof(float);
+  TORCH_CHECK(lds <= 64 * 1024,
+              "seqmix: attention head sizes exceed the LDS budget");
+  const bool vec = (dk * sizeof(T)) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(kcache.data_ptr()) % 16 == 0;
+#define LAUNCH_ATT(GS_, VEC_)                                               \
+  hipLaunchKernelGGL((biased_attention_kernel<T, GS_, VEC_>),               \
+      dim3(T_, H / GS_), dim3(256), lds, cur_stream(), ptr<T>(out),         \
+      cptr<T>(proj), (int)proj.stride(0), (int)off_q, cptr<T>(kcache),      \
+      cptr<T>(vcache), cptr<int>(page_table), (int)page_table.stride(0),    \
+      cptr<int>(tok_seq), cptr<int>(positions), cptr<int>(seq_len),         \
+      r1 ? cptr<float>(*r1) : nullptr, r2 ? cptr<float>(*r2) : nullptr, H,  \
+      G, dk, dv, ps, (float)scale, (float)temp_coef, (int)temp_every,       \
+      r1 ? 1 : 0)
+  if (GS == 4) { if (vec) LAUNCH_ATT(4, true); else LAUNCH_ATT(4, false); }
+  else if (GS == 2) { if (vec) LAUNCH_ATT(2, true); else LAUNCH_ATT(2, false); }
+  else { if (vec) LAUNCH_ATT(1, true); else LAUNCH_ATT(1, false); }
+#undef LAUNCH_ATT
 }
 
 }  // namespace
@@ -178,12 +333,7 @@ void biased_attention(torch::Tensor out, torch::Tensor proj, int64_t off_q,
               "bias parameters");
   SEQ_CHECK(temp_every >= 1, "temperature period");
   if (T_ == 0) return;
-  DISPATCH_ACT(proj, hipLaunchKernelGGL(
-      biased_attention_kernel<T>, dim3(T_, H), dim3(64), dk * sizeof(float),
-      cur_stream(), ptr<T>(out), cptr<T>(proj), (int)proj.stride(0),
-      (int)off_q, cptr<T>(kcache), cptr<T>(vcache), cptr<int>(page_table),
-      (int)page_table.stride(0), cptr<int>(tok_seq), cptr<int>(positions),
-      cptr<int>(seq_len), r1 ? cptr<float>(*r1) : nullptr,
-      r2 ? cptr<float>(*r2) : nullptr, H, G, dk, dv, ps, (float)scale,
-      (float)temp_coef, (int)temp_every, r1 ? 1 : 0););
+  DISPATCH_ACT(proj, launch_attention<T>(
+      out, proj, off_q, kcache, vcache, page_table, tok_seq, positions,
+      seq_len, r1, r2, scale, temp_coef, temp_every););
 }

@@ -9,11 +9,18 @@
 // JW = 64 / KP) share a column and reduce their partial dot products with
 // lane shuffles. R <= RMAX and KP is a power of two, so dk <= RMAX * 64.
 // State is fp32 in HBM, loaded once per step and stored once.
+//
+// The walk over a portion is latency bound (one token depends on the one
+// before), so each token's inputs are fetched into registers one token
+// ahead, and the key-side vectors go through a double-buffered LDS stage:
+// one barrier per token, global latency hidden behind the previous token's
+// arithmetic.
 #include "seq_common.h"
 
 namespace {
 
 constexpr int RMAX = 32;
+constexpr int PEMAX = 4;  // staged elements per thread and vector
 
 struct SeqArgs {
   const int* seq_start;
@@ -35,6 +42,9 @@ inline Geometry geometry(int dk, int dv) {
   g.JW = 64 / g.KP;
   const int waves = (dv + g.JW - 1) / g.JW;
   g.NW = waves < 4 ? waves : 4;
+  // enough threads to stage a key-side vector with PEMAX elements each
+  const int need = (dk + 64 * PEMAX - 1) / (64 * PEMAX);
+  if (g.NW < need) g.NW = need;
   g.tiles = (waves + g.NW - 1) / g.NW;
   return g;
 }
@@ -64,13 +74,13 @@ DEVINL float part_sum(float x, int JW) {
 template <typename T>
 __global__ void gated_delta_kernel(
     float* __restrict__ out,          // [T, H, dv]
-    const float* __restrict__ qkv,    // [T, Cq + Ck + Cv] after conv + silu
+    const float* __restrict__ qkv,    // [T, Cq + Ck + Cv]: unit k, scaled
+                                      // unit q, v (after conv + silu)
     const T* __restrict__ proj, int proj_stride, int off_b, int off_a,
     const float* __restrict__ A_log, const float* __restrict__ dt_bias,
     float* __restrict__ state,        // [slots, H, dk, dv]
-    SeqArgs sa, int H, int G, int dk, int dv, int KP, int R, float qscale,
-    float unit_eps) {
-  extern __shared__ float lds[];  // [2][dk]: unit k, scaled unit q
+    SeqArgs sa, int H, int G, int dk, int dv, int KP, int R) {
+  extern __shared__ float lds[];  // [2 buffers][k | q][dk]
   const int s = blockIdx.x, hh = blockIdx.y;
   const int len = sa.seq_len[s];
   if (len == 0) return;
@@ -85,37 +95,42 @@ __global__ void gated_delta_kernel(
   const int kvh = hh / (H / G);
   const int Cq = G * dk, Cc = 2 * G * dk + H * dv;
   float* sbase = state + ((int64_t)sa.seq_slot[s] * H + hh) * dk * dv;
-  float* kl = lds;
-  float* ql = lds + dk;
   float S[RMAX];
   LOAD_STATE(S, sbase, fresh)
   const float a_neg = -expf(A_log[hh]);
   const float dtb = dt_bias[hh];
 
-  for (int t = start; t < start + len; t++) {
+  // inputs of the token about to be processed, fetched one token ahead
+  float kpre[PEMAX], qpre[PEMAX], braw, araw, vj;
+  auto fetch = [&](int t) {
     const float* row = qkv + (int64_t)t * Cc;
-    // every wave normalises redundantly; wave 0 publishes
-    float sq = 0.f, sk = 0.f;
-    for (int i = lane; i < dk; i += 64) {
-      const float qv = row[kvh * dk + i], kv = row[Cq + kvh * dk + i];
-      sq += qv * qv;
-      sk += kv * kv;
+#pragma unroll
+    for (int e = 0; e < PEMAX; e++) {
+      const int i = threadIdx.x + e * blockDim.x;
+      kpre[e] = i < dk ? row[Cq + kvh * dk + i] : 0.f;
+      qpre[e] = i < dk ? row[kvh * dk + i] : 0.f;
     }
-    sq = wave_sum(sq);
-    sk = wave_sum(sk);
-    const float qn = qscale / sqrtf(sq + unit_eps);
-    const float kn = 1.f / sqrtf(sk + unit_eps);
-    __syncthreads();  // previous token's readers are done
-    for (int i = threadIdx.x; i < dk; i += blockDim.x) {
-      kl[i] = row[Cq + kvh * dk + i] * kn;
-      ql[i] = row[kvh * dk + i] * qn;
+    braw = to_f(proj[(int64_t)t * proj_stride + off_b + hh]);
+    araw = to_f(proj[(int64_t)t * proj_stride + off_a + hh]);
+    vj = valid ? row[2 * Cq + hh * dv + j] : 0.f;
+  };
+  fetch(start);
+  for (int t = start; t < start + len; t++) {
+    float* kl = lds + ((t - start) & 1) * 2 * dk;
+    float* ql = kl + dk;
+#pragma unroll
+    for (int e = 0; e < PEMAX; e++) {
+      const int i = threadIdx.x + e * blockDim.x;
+      if (i < dk) {
+        kl[i] = kpre[e];
+        ql[i] = qpre[e];
+      }
     }
-    __syncthreads();
-    const float braw = to_f(proj[(int64_t)t * proj_stride + off_b + hh]);
-    const float araw = to_f(proj[(int64_t)t * proj_stride + off_a + hh]);
     const float beta = sigmoid_f(braw);
     const float g = expf(a_neg * softplus_f(araw + dtb));
-    const float vj = valid ? row[2 * Cq + hh * dv + j] : 0.f;
+    const float v_cur = vj;
+    __syncthreads();
+    if (t + 1 < start + len) fetch(t + 1);
     float dot = 0.f;
 #pragma unroll
     for (int r = 0; r < RMAX; r++) {
@@ -126,7 +141,7 @@ __global__ void gated_delta_kernel(
       }
     }
     dot = part_sum(dot, JW);
-    const float u = beta * (vj - dot);
+    const float u = beta * (v_cur - dot);
     float o = 0.f;
 #pragma unroll
     for (int r = 0; r < RMAX; r++) {
@@ -142,6 +157,20 @@ __global__ void gated_delta_kernel(
   STORE_STATE(S, sbase)
 }
 
+// q and k of the delta rule become unit vectors per head, in place:
+// x / sqrt(sum(x^2) + unit_eps), q also times qscale. One wave per
+// (token, q-or-k head).
+__global__ void unit_heads_kernel(float* __restrict__ qkv, int Cc, int G,
+                                  int dk, float qscale, float unit_eps) {
+  const int t = blockIdx.x, v = blockIdx.y, lane = threadIdx.x;
+  float* x = qkv + (int64_t)t * Cc + v * dk;  // q heads, then k heads
+  float ss = 0.f;
+  for (int i = lane; i < dk; i += 64) ss += x[i] * x[i];
+  ss = wave_sum(ss);
+  const float mul = (v < G ? qscale : 1.f) / sqrtf(ss + unit_eps);
+  for (int i = lane; i < dk; i += 64) x[i] *= mul;
+}
+
 // ---------------------------------------------------------------------------
 // RWKV-style time mixing. Per token, with w = exp(-exp(wraw + w0)):
 // o = (S + diag(u) k v^T)^T r; S <- diag(w) S + k v^T.
@@ -155,7 +184,7 @@ __global__ void rwkv_kernel(
     const float* __restrict__ u,   // [H, d]
     float* __restrict__ state,     // [slots, H, d, d]
     SeqArgs sa, int H, int dk, int dv, int KP, int R) {
-  extern __shared__ float lds[];  // [3][dk]: r, k, w
+  extern __shared__ float lds[];  // [2 buffers][r | k | w][dk]
   const int s = blockIdx.x, hh = blockIdx.y;
   const int len = sa.seq_len[s];
   if (len == 0) return;
@@ -168,9 +197,6 @@ __global__ void rwkv_kernel(
   const int j = (blockIdx.z * nw + wave) * JW + (lane % JW);
   const bool valid = j < dv;
   float* sbase = state + ((int64_t)sa.seq_slot[s] * H + hh) * dk * dv;
-  float* rl = lds;
-  float* kl = lds + dk;
-  float* wl = lds + 2 * dk;
   float S[RMAX], U[RMAX];
   LOAD_STATE(S, sbase, fresh)
 #pragma unroll
@@ -178,23 +204,48 @@ __global__ void rwkv_kernel(
     const int rowi = part * R + r;
     U[r] = (r < R && rowi < dk) ? u[hh * dk + rowi] : 0.f;
   }
+  float w0r[PEMAX];
+#pragma unroll
+  for (int e = 0; e < PEMAX; e++) {
+    const int i = threadIdx.x + e * blockDim.x;
+    w0r[e] = i < dk ? w0[hh * dk + i] : 0.f;
+  }
   const int HD = H * dk;
-  for (int t = start; t < start + len; t++) {
+  float rpre[PEMAX], kpre[PEMAX], wpre[PEMAX], vj;
+  auto fetch = [&](int t) {
     const int64_t base = (int64_t)t * HD + hh * dk;
-    __syncthreads();
-    for (int i = threadIdx.x; i < dk; i += blockDim.x) {
-      rl[i] = to_f(r_[base + i]);
-      kl[i] = to_f(k_[base + i]);
-      wl[i] = expf(-expf(to_f(wraw[base + i]) + w0[hh * dk + i]));
+#pragma unroll
+    for (int e = 0; e < PEMAX; e++) {
+      const int i = threadIdx.x + e * blockDim.x;
+      rpre[e] = i < dk ? to_f(r_[base + i]) : 0.f;
+      kpre[e] = i < dk ? to_f(k_[base + i]) : 0.f;
+      wpre[e] = i < dk ? to_f(wraw[base + i]) : 0.f;
     }
+    vj = valid ? to_f(v_[(int64_t)t * H * dv + hh * dv + j]) : 0.f;
+  };
+  fetch(start);
+  for (int t = start; t < start + len; t++) {
+    float* rl = lds + ((t - start) & 1) * 3 * dk;
+    float* kl = rl + dk;
+    float* wl = rl + 2 * dk;
+#pragma unroll
+    for (int e = 0; e < PEMAX; e++) {
+      const int i = threadIdx.x + e * blockDim.x;
+      if (i < dk) {
+        rl[i] = rpre[e];
+        kl[i] = kpre[e];
+        wl[i] = expf(-expf(wpre[e] + w0r[e]));
+      }
+    }
+    const float v_cur = vj;
     __syncthreads();
-    const float vj = valid ? to_f(v_[(int64_t)t * H * dv + hh * dv + j]) : 0.f;
+    if (t + 1 < start + len) fetch(t + 1);
     float o = 0.f;
 #pragma unroll
     for (int r = 0; r < RMAX; r++) {
       const int rowi = part * R + r;
       if (r < R && rowi < dk) {
-        const float kv = kl[rowi] * vj;
+        const float kv = kl[rowi] * v_cur;
         o += rl[rowi] * (S[r] + U[r] * kv);
         S[r] = wl[rowi] * S[r] + kv;
       }
@@ -221,7 +272,7 @@ __global__ void mlstm_kernel(
     const float* __restrict__ state_m,  // [slots, H]
     SeqArgs sa, int H, int dk, int dv, int KP, int R, float qscale, float cap,
     float den_eps) {
-  extern __shared__ float lds[];  // [2][dk]: k, q
+  extern __shared__ float lds[];  // [2 buffers][k | q][dk]
   const int s = blockIdx.x, hh = blockIdx.y;
   const int len = sa.seq_len[s];
   if (len == 0) return;
@@ -236,8 +287,6 @@ __global__ void mlstm_kernel(
   const int slot = sa.seq_slot[s];
   float* sbase = state_S + ((int64_t)slot * H + hh) * dk * dv;
   const float* nbase = state_n + ((int64_t)slot * H + hh) * dk;
-  float* kl = lds;
-  float* ql = lds + dk;
   float S[RMAX], N[RMAX];
   LOAD_STATE(S, sbase, fresh)
 #pragma unroll
@@ -248,27 +297,46 @@ __global__ void mlstm_kernel(
   float m = fresh ? 0.f : state_m[slot * H + hh];
   const float ib = i_bias[hh], fb = f_bias[hh];
 
-  for (int t = start; t < start + len; t++) {
+  float kpre[PEMAX], qpre[PEMAX], iraw, fraw, vj;
+  auto fetch = [&](int t) {
     const T* row = proj + (int64_t)t * proj_stride;
-    __syncthreads();
-    for (int i = threadIdx.x; i < dk; i += blockDim.x) {
-      kl[i] = to_f(row[off_k + hh * dk + i]);
-      ql[i] = to_f(row[off_q + hh * dk + i]) * qscale;
+#pragma unroll
+    for (int e = 0; e < PEMAX; e++) {
+      const int i = threadIdx.x + e * blockDim.x;
+      kpre[e] = i < dk ? to_f(row[off_k + hh * dk + i]) : 0.f;
+      qpre[e] = i < dk ? to_f(row[off_q + hh * dk + i]) * qscale : 0.f;
     }
+    iraw = to_f(row[off_i + hh]);
+    fraw = to_f(row[off_f + hh]);
+    vj = valid ? to_f(row[off_v + hh * dv + j]) : 0.f;
+  };
+  fetch(start);
+  for (int t = start; t < start + len; t++) {
+    float* kl = lds + ((t - start) & 1) * 2 * dk;
+    float* ql = kl + dk;
+#pragma unroll
+    for (int e = 0; e < PEMAX; e++) {
+      const int i = threadIdx.x + e * blockDim.x;
+      if (i < dk) {
+        kl[i] = kpre[e];
+        ql[i] = qpre[e];
+      }
+    }
+    const float ig = cap * tanhf((iraw + ib) / cap);
+    const float fg = logsigmoid_f(cap * tanhf((fraw + fb) / cap));
+    const float v_cur = vj;
     __syncthreads();
-    const float ig = cap * tanhf((to_f(row[off_i + hh]) + ib) / cap);
-    const float fg = logsigmoid_f(cap * tanhf((to_f(row[off_f + hh]) + fb) / cap));
+    if (t + 1 < start + len) fetch(t + 1);
     const float mn = fmaxf(fg + m, ig);
     const float a = expf(fg + m - mn), b = expf(ig - mn);
     m = mn;
-    const float vj = valid ? to_f(row[off_v + hh * dv + j]) : 0.f;
     float num = 0.f, nq = 0.f;
 #pragma unroll
     for (int r = 0; r < RMAX; r++) {
       const int rowi = part * R + r;
       if (r < R && rowi < dk) {
         const float bk = b * kl[rowi];
-        S[r] = a * S[r] + bk * vj;
+        S[r] = a * S[r] + bk * v_cur;
         N[r] = a * N[r] + bk;
         num += S[r] * ql[rowi];
         nq += N[r] * ql[rowi];
@@ -335,6 +403,7 @@ SeqArgs seq_args(const torch::Tensor& seq_start, const torch::Tensor& seq_len,
 
 }  // namespace
 
+// qkv holds q | k | v after the convolution; q and k are normalised in place
 void gated_delta_rule(torch::Tensor out, torch::Tensor qkv, torch::Tensor proj,
                       int64_t off_b, int64_t off_a, torch::Tensor A_log,
                       torch::Tensor dt_bias, torch::Tensor state,
@@ -360,12 +429,15 @@ void gated_delta_rule(torch::Tensor out, torch::Tensor qkv, torch::Tensor proj,
   if (T_ == 0 || B == 0) return;
   SeqArgs sa = seq_args(seq_start, seq_len, seq_slot, seq_pos0, state.size(0));
   Geometry g = geometry(dk, dv);
+  hipLaunchKernelGGL(unit_heads_kernel, dim3(T_, 2 * (int)G), dim3(64), 0,
+                     cur_stream(), ptr<float>(qkv), (int)qkv.size(1), (int)G,
+                     dk, (float)qscale, (float)unit_eps);
   DISPATCH_ACT(proj, hipLaunchKernelGGL(
       gated_delta_kernel<T>, dim3(B, H, g.tiles), dim3(g.NW * 64),
-      2 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<float>(qkv),
+      4 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<float>(qkv),
       cptr<T>(proj), (int)proj.stride(0), (int)off_b, (int)off_a,
       cptr<float>(A_log), cptr<float>(dt_bias), ptr<float>(state), sa, H,
-      (int)G, dk, dv, g.KP, g.R, (float)qscale, (float)unit_eps););
+      (int)G, dk, dv, g.KP, g.R););
 }
 
 void rwkv_time_mix(torch::Tensor out, torch::Tensor r, torch::Tensor k,
@@ -392,7 +464,7 @@ void rwkv_time_mix(torch::Tensor out, torch::Tensor r, torch::Tensor k,
   Geometry g = geometry(dk, dv);
   DISPATCH_ACT(r, hipLaunchKernelGGL(
       rwkv_kernel<T>, dim3(B, H, g.tiles), dim3(g.NW * 64),
-      3 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(r),
+      6 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(r),
       cptr<T>(k), cptr<T>(v), cptr<T>(wraw), cptr<float>(w0), cptr<float>(u),
       ptr<float>(state), sa, H, dk, dv, g.KP, g.R););
 }
@@ -429,7 +501,7 @@ void mlstm_memory(torch::Tensor out, torch::Tensor proj, int64_t off_q,
   Geometry g = geometry(dk, dv);
   DISPATCH_ACT(proj, hipLaunchKernelGGL(
       mlstm_kernel<T>, dim3(B, H, g.tiles), dim3(g.NW * 64),
-      2 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(proj),
+      4 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(proj),
       (int)proj.stride(0), (int)off_q, (int)off_k, (int)off_v, (int)off_i,
       (int)off_f, cptr<float>(i_bias), cptr<float>(f_bias),
       ptr<float>(state_S), ptr<float>(state_n), ptr<float>(state_m), sa, H, dk,
