@@ -65,17 +65,19 @@ template <> struct Vec16<bf16_t> {
   }
 };
 
-// One workgroup (4 waves) per (token row, group of GS query heads that
-// share a kv head). The waves take 64-key chunks in turn and are merged
-// through LDS at the end, so a decoded token with a long context still
-// spreads over 4 waves. Within a chunk, 4 adjacent lanes share a key:
-// each reads every 4th 16-byte piece of the key row (a quad covers 64
-// contiguous bytes) and the quad adds its partial dots, 16 keys a pass, 4
-// passes a chunk; no transposed staging is needed. For the weighted sum
-// lanes own value channels and read value rows as they lie in the page.
-// VEC is off when a key row is not a whole number of 16-byte pieces.
-template <typename T, int GS, bool VEC>
-__global__ __launch_bounds__(256) void biased_attention_kernel(
+// One workgroup per (token row, group of GS query heads that share a kv
+// head). Its waves (4 for large prompt batches, 16 when few rows are in
+// flight, so a decoded token with a long context still fills a CU) take
+// 64-key chunks in turn and are merged through LDS at the end. Within a
+// chunk, 4 adjacent lanes share a key: each reads every 4th 16-byte piece
+// of the key row (a quad covers 64 contiguous bytes) and the quad adds its
+// partial dots, 16 keys a pass, 4 passes a chunk; no transposed staging is
+// needed. For the weighted sum a lane owns pairs of adjacent value channels
+// and reads value rows as they lie in the page, eight rows in flight.
+// VEC is off when a key row is not a whole number of 16-byte pieces; EVT
+// is the number of value channels a lane owns.
+template <typename T, int GS, bool VEC, int EVT>
+__global__ __launch_bounds__(1024) void biased_attention_kernel(
     T* __restrict__ out,  // [T, H, dv]
     const T* __restrict__ proj, int proj_stride, int off_q,
     const T* __restrict__ kcache, const T* __restrict__ vcache,
@@ -84,9 +86,11 @@ __global__ __launch_bounds__(256) void biased_attention_kernel(
     const int* __restrict__ seq_len, const float* __restrict__ r1,
     const float* __restrict__ r2, int H, int G, int dk, int dv, int ps,
     float scale, float temp_coef, int temp_every, int has_bias) {
-  extern __shared__ float lds[];  // q [GS][dk]; merge [4][GS][2 + dv]
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  // q [GS][dk]; merge [waves][GS][2 + dv]
   constexpr int VN = Vec16<T>::N;
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nwv = blockDim.x >> 6;
   const int s = tok_seq[t];
   if (seq_len[s] == 0) return;  // padding row
   const int h0 = blockIdx.y * GS;  // first query head of this group
@@ -98,7 +102,7 @@ __global__ __launch_bounds__(256) void biased_attention_kernel(
   const float qmul = temp * scale;
   float* qs = lds;
   float* mg = lds + GS * dk;
-  for (int i = threadIdx.x; i < GS * dk; i += 256)
+  for (int i = threadIdx.x; i < GS * dk; i += blockDim.x)
     qs[i] = to_f(proj[(int64_t)t * proj_stride + off_q + h0 * dk + i]) * qmul;
   __syncthreads();
   const int* table = page_table + (int64_t)s * table_stride;
@@ -109,19 +113,23 @@ __global__ __launch_bounds__(256) void biased_attention_kernel(
     b2[a] = has_bias ? r2[h0 + a] : 0.f;
   }
   const int quad = lane >> 2, qq = lane & 3;
-  const int nvec = dk / VN;  // used when VEC
+  const int nvec = dk / VN;        // used when VEC
+  const bool run16 = ps % 16 == 0;  // a 16-key pass lies in one page
+  // adjacent channels load as one word when rows stay aligned
+  const bool pair = (dv & 1) == 0 &&
+                    reinterpret_cast<uintptr_t>(vcache) % 8 == 0;
 
-  float m[GS], l[GS], acc[GS][EVMAX];
+  float m[GS], l[GS], acc[GS][EVT];
 #pragma unroll
   for (int a = 0; a < GS; a++) {
     m[a] = -INFINITY;
     l[a] = 0.f;
 #pragma unroll
-    for (int e = 0; e < EVMAX; e++) acc[a][e] = 0.f;
+    for (int e = 0; e < EVT; e++) acc[a][e] = 0.f;
   }
   const int ctx = pos + 1;
   const int nchunks = (ctx + 63) >> 6;
-  for (int c = wave; c < nchunks; c += 4) {
+  for (int c = wave; c < nchunks; c += nwv) {
     const int j0 = c << 6;
     // ---- scores: pass p covers keys j0 + 16 p + quad ----
     float sc[4][GS];
@@ -135,14 +143,29 @@ __global__ __launch_bounds__(256) void biased_attention_kernel(
         const int64_t page = table[j / ps];
         const T* k = kcache + ((page * G + g) * ps + (j % ps)) * dk;
         if (VEC) {
-          for (int v = qq; v < nvec; v += 4) {
-            Vec16<T> kv;
-            kv.v = *reinterpret_cast<const decltype(kv.v)*>(k + v * VN);
+          for (int v0 = qq; v0 < nvec; v0 += 16) {
+            Vec16<T> kv[4];
 #pragma unroll
-            for (int i = 0; i < VN; i++) {
-              const float kf = kv.get(i);
+            for (int u = 0; u < 4; u++)
+              if (v0 + 4 * u < nvec)
+                kv[u].v = *reinterpret_cast<const decltype(kv[u].v)*>(
+                    k + (v0 + 4 * u) * VN);
 #pragma unroll
-              for (int a = 0; a < GS; a++) d[a] += qs[a * dk + v * VN + i] * kf;
+            for (int u = 0; u < 4; u++) {
+              const int v = v0 + 4 * u;
+              if (v < nvec) {
+#pragma unroll
+                for (int a = 0; a < GS; a++) {
+                  const float4* q4 =
+                      reinterpret_cast<const float4*>(qs + a * dk + v * VN);
+#pragma unroll
+                  for (int i4 = 0; i4 < VN / 4; i4++) {
+                    const float4 q = q4[i4];
+                    d[a] += q.x * kv[u].get(4 * i4) + q.y * kv[u].get(4 * i4 + 1) +
+                            q.z * kv[u].get(4 * i4 + 2) + q.w * kv[u].get(4 * i4 + 3);
+                  }
+                }
+              }
             }
           }
         } else {
@@ -182,32 +205,76 @@ __global__ __launch_bounds__(256) void biased_attention_kernel(
       l[a] = l[a] * corr + 0.25f * wave_sum(sum);  // 4 lanes per key
       m[a] = mx;
 #pragma unroll
-      for (int e = 0; e < EVMAX; e++) acc[a][e] *= corr;
+      for (int e = 0; e < EVT; e++) acc[a][e] *= corr;
     }
-    // ---- weighted sum of values: lanes own channels ----
+    // ---- weighted sum of values: lane owns channels
+    //      (e / 2) * 128 + 2 * lane + (e & 1) ----
 #pragma unroll
     for (int p = 0; p < 4; p++) {
-      const int nk = min(16, ctx - (j0 + 16 * p));
-      for (int kk = 0; kk < nk; kk++) {
-        const int j = j0 + 16 * p + kk;
-        const int64_t page = table[j / ps];
-        const T* v = vcache + ((page * G + g) * ps + (j % ps)) * dv;
-        float w[GS];
+      const int jp = j0 + 16 * p;
+      const int nk = min(16, ctx - jp);
+      if (nk <= 0) break;
+      const T* vrun = nullptr;
+      if (run16)
+        vrun = vcache + (((int64_t)table[jp / ps] * G + g) * ps + (jp % ps)) * dv;
+      for (int k0 = 0; k0 < nk; k0 += 8) {
+        float vf[8][EVT];
 #pragma unroll
-        for (int a = 0; a < GS; a++) w[a] = __shfl(pr[p][a], kk << 2, 64);
+        for (int u = 0; u < 8; u++) {
+          const int kk = k0 + u;
+          if (kk < nk) {
+            const T* v;
+            if (run16) {
+              v = vrun + (int64_t)kk * dv;
+            } else {
+              const int j = jp + kk;
+              v = vcache + (((int64_t)table[j / ps] * G + g) * ps + (j % ps)) * dv;
+            }
 #pragma unroll
-        for (int e = 0; e < EVMAX; e++) {
-          const int ch = lane + 64 * e;
-          if (ch < dv) {
-            const float vf = to_f(v[ch]);
+            for (int e = 0; e < EVT; e += 2) {
+              const int ch = (e / 2) * 128 + 2 * lane;
+              if (pair) {
+                if (ch < dv) {  // dv even: ch + 1 < dv as well
+                  if (sizeof(T) == 2) {
+                    const uint32_t w = *reinterpret_cast<const uint32_t*>(v + ch);
+                    union { float f; uint32_t u; } c0, c1;
+                    c0.u = w << 16;
+                    c1.u = w & 0xffff0000u;
+                    vf[u][e] = c0.f;
+                    if (e + 1 < EVT) vf[u][e + 1] = c1.f;
+                  } else {
+                    const float2 w = *reinterpret_cast<const float2*>(v + ch);
+                    vf[u][e] = w.x;
+                    if (e + 1 < EVT) vf[u][e + 1] = w.y;
+                  }
+                } else {
+                  vf[u][e] = 0.f;
+                  if (e + 1 < EVT) vf[u][e + 1] = 0.f;
+                }
+              } else {
+                vf[u][e] = ch < dv ? to_f(v[ch]) : 0.f;
+                if (e + 1 < EVT) vf[u][e + 1] = ch + 1 < dv ? to_f(v[ch + 1]) : 0.f;
+              }
+            }
+          } else {
 #pragma unroll
-            for (int a = 0; a < GS; a++) acc[a][e] += w[a] * vf;
+            for (int e = 0; e < EVT; e++) vf[u][e] = 0.f;
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const int src = ((k0 + u) & 15) << 2;  // lane that holds this key
+#pragma unroll
+          for (int a = 0; a < GS; a++) {
+            const float w = __shfl(pr[p][a], src, 64);
+#pragma unroll
+            for (int e = 0; e < EVT; e++) acc[a][e] += w * vf[u][e];
           }
         }
       }
     }
   }
-  // ---- merge the 4 waves ----
+  // ---- merge the waves ----
   const int MS = 2 + dv;  // floats per (wave, head) record
 #pragma unroll
   for (int a = 0; a < GS; a++) {
@@ -217,25 +284,27 @@ __global__ __launch_bounds__(256) void biased_attention_kernel(
       rec[1] = l[a];
     }
 #pragma unroll
-    for (int e = 0; e < EVMAX; e++) {
-      const int ch = lane + 64 * e;
+    for (int e = 0; e < EVT; e++) {
+      const int ch = (e / 2) * 128 + 2 * lane + (e & 1);
       if (ch < dv) rec[2 + ch] = acc[a][e];
     }
   }
   __syncthreads();
-  for (int a = wave; a < GS; a += 4) {  // wave a finishes head a
+  for (int a = wave; a < GS; a += nwv) {  // wave a finishes head a
     float mx = -INFINITY;
-    for (int w = 0; w < 4; w++) mx = fmaxf(mx, mg[(w * GS + a) * MS]);
-    float lt = 0.f, f[4];
-    for (int w = 0; w < 4; w++) {
+    for (int w = 0; w < nwv; w++) mx = fmaxf(mx, mg[(w * GS + a) * MS]);
+    float lt = 0.f;
+    for (int w = 0; w < nwv; w++) {
       const float mw = mg[(w * GS + a) * MS];
-      f[w] = (mw == -INFINITY) ? 0.f : expf(mw - mx);
-      lt += f[w] * mg[(w * GS + a) * MS + 1];
+      if (mw != -INFINITY) lt += expf(mw - mx) * mg[(w * GS + a) * MS + 1];
     }
     const float inv = 1.f / lt;
     for (int ch = lane; ch < dv; ch += 64) {
       float o = 0.f;
-      for (int w = 0; w < 4; w++) o += f[w] * mg[(w * GS + a) * MS + 2 + ch];
+      for (int w = 0; w < nwv; w++) {
+        const float mw = mg[(w * GS + a) * MS];
+        if (mw != -INFINITY) o += expf(mw - mx) * mg[(w * GS + a) * MS + 2 + ch];
+      }
       out[((int64_t)t * H + h0 + a) * dv + ch] = from_f<T>(o * inv);
     }
   }
@@ -253,23 +322,34 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
   const int G = kcache.size(1), ps = kcache.size(2), dk = kcache.size(3);
   const int gsz = H / G;
   const int GS = gsz % 4 == 0 ? 4 : (gsz % 2 == 0 ? 2 : 1);
-  const size_t lds = (size_t)(GS * dk + 4 * GS * (2 + dv)) * sizeof(float);
+  // few rows in flight (decoding): 16 waves split the keys of each row
+  const int NW = T_ * (H / GS) <= 2048 ? 16 : 4;
+  const size_t lds = (size_t)(GS * dk + NW * GS * (2 + dv)) * sizeof(float);
   TORCH_CHECK(lds <= 64 * 1024,
               "seqmix: attention head sizes exceed the LDS budget");
   const bool vec = (dk * sizeof(T)) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(kcache.data_ptr()) % 16 == 0;
-#define LAUNCH_ATT(GS_, VEC_)                                               \
-  hipLaunchKernelGGL((biased_attention_kernel<T, GS_, VEC_>),               \
-      dim3(T_, H / GS_), dim3(256), lds, cur_stream(), ptr<T>(out),         \
+  const bool small = dv <= 128;
+#define LAUNCH_ATT(GS_, VEC_, EVT_)                                         \
+  hipLaunchKernelGGL((biased_attention_kernel<T, GS_, VEC_, EVT_>),         \
+      dim3(T_, H / GS_), dim3(NW * 64), lds, cur_stream(), ptr<T>(out),     \
       cptr<T>(proj), (int)proj.stride(0), (int)off_q, cptr<T>(kcache),      \
       cptr<T>(vcache), cptr<int>(page_table), (int)page_table.stride(0),    \
       cptr<int>(tok_seq), cptr<int>(positions), cptr<int>(seq_len),         \
       r1 ? cptr<float>(*r1) : nullptr, r2 ? cptr<float>(*r2) : nullptr, H,  \
       G, dk, dv, ps, (float)scale, (float)temp_coef, (int)temp_every,       \
       r1 ? 1 : 0)
-  if (GS == 4) { if (vec) LAUNCH_ATT(4, true); else LAUNCH_ATT(4, false); }
-  else if (GS == 2) { if (vec) LAUNCH_ATT(2, true); else LAUNCH_ATT(2, false); }
-  else { if (vec) LAUNCH_ATT(1, true); else LAUNCH_ATT(1, false); }
+#define LAUNCH_GS(GS_)                                                      \
+  do {                                                                      \
+    if (vec && small) LAUNCH_ATT(GS_, true, 2);                             \
+    else if (vec) LAUNCH_ATT(GS_, true, EVMAX);                             \
+    else if (small) LAUNCH_ATT(GS_, false, 2);                              \
+    else LAUNCH_ATT(GS_, false, EVMAX);                                     \
+  } while (0)
+  if (GS == 4) LAUNCH_GS(4);
+  else if (GS == 2) LAUNCH_GS(2);
+  else LAUNCH_GS(1);
+#undef LAUNCH_GS
 #undef LAUNCH_ATT
 }
 

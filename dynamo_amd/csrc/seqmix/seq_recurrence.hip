@@ -11,16 +11,19 @@
 // State is fp32 in HBM, loaded once per step and stored once.
 //
 // The walk over a portion is latency bound (one token depends on the one
-// before), so each token's inputs are fetched into registers one token
-// ahead, and the key-side vectors go through a double-buffered LDS stage:
-// one barrier per token, global latency hidden behind the previous token's
-// arithmetic.
+// before, and every token's inputs lie in another page of the projection
+// buffers), so each token's inputs are fetched into a ring of registers
+// DEPTH tokens ahead, and the key-side vectors go through a double-buffered
+// LDS stage: one barrier per token, global latency spread over DEPTH
+// tokens' arithmetic. PE is the number of staged elements a thread carries
+// per key-side vector (1 when the workgroup is at least dk threads).
 #include "seq_common.h"
 
 namespace {
 
 constexpr int RMAX = 32;
 constexpr int PEMAX = 4;  // staged elements per thread and vector
+constexpr int DEPTH = 4;  // tokens fetched ahead
 
 struct SeqArgs {
   const int* seq_start;
@@ -71,8 +74,8 @@ DEVINL float part_sum(float x, int JW) {
 // Gated delta rule. Per token: S <- g S; u = beta (v - S^T k);
 // S <- S + k u^T; o = S^T q. q and k arrive after the short convolution and
 // are made unit vectors here (q also scaled by qscale).
-template <typename T>
-__global__ void gated_delta_kernel(
+template <typename T, int PE>
+__global__ __launch_bounds__(512) void gated_delta_kernel(
     float* __restrict__ out,          // [T, H, dv]
     const float* __restrict__ qkv,    // [T, Cq + Ck + Cv]: unit k, scaled
                                       // unit q, v (after conv + silu)
@@ -100,59 +103,67 @@ __global__ void gated_delta_kernel(
   const float a_neg = -expf(A_log[hh]);
   const float dtb = dt_bias[hh];
 
-  // inputs of the token about to be processed, fetched one token ahead
-  float kpre[PEMAX], qpre[PEMAX], braw, araw, vj;
-  auto fetch = [&](int t) {
+  struct In { float k[PE], q[PE], braw, araw, vj; };
+  In pre[DEPTH];
+  const int end = start + len;
+  auto fetch = [&](In& in, int t) {
     const float* row = qkv + (int64_t)t * Cc;
 #pragma unroll
-    for (int e = 0; e < PEMAX; e++) {
+    for (int e = 0; e < PE; e++) {
       const int i = threadIdx.x + e * blockDim.x;
-      kpre[e] = i < dk ? row[Cq + kvh * dk + i] : 0.f;
-      qpre[e] = i < dk ? row[kvh * dk + i] : 0.f;
+      in.k[e] = i < dk ? row[Cq + kvh * dk + i] : 0.f;
+      in.q[e] = i < dk ? row[kvh * dk + i] : 0.f;
     }
-    braw = to_f(proj[(int64_t)t * proj_stride + off_b + hh]);
-    araw = to_f(proj[(int64_t)t * proj_stride + off_a + hh]);
-    vj = valid ? row[2 * Cq + hh * dv + j] : 0.f;
+    in.braw = to_f(proj[(int64_t)t * proj_stride + off_b + hh]);
+    in.araw = to_f(proj[(int64_t)t * proj_stride + off_a + hh]);
+    in.vj = valid ? row[2 * Cq + hh * dv + j] : 0.f;
   };
-  fetch(start);
-  for (int t = start; t < start + len; t++) {
-    float* kl = lds + ((t - start) & 1) * 2 * dk;
-    float* ql = kl + dk;
 #pragma unroll
-    for (int e = 0; e < PEMAX; e++) {
-      const int i = threadIdx.x + e * blockDim.x;
-      if (i < dk) {
-        kl[i] = kpre[e];
-        ql[i] = qpre[e];
-      }
-    }
-    const float beta = sigmoid_f(braw);
-    const float g = expf(a_neg * softplus_f(araw + dtb));
-    const float v_cur = vj;
-    __syncthreads();
-    if (t + 1 < start + len) fetch(t + 1);
-    float dot = 0.f;
+  for (int u = 0; u < DEPTH; u++)
+    if (start + u < end) fetch(pre[u], start + u);
+  for (int t0 = start; t0 < end; t0 += DEPTH) {
 #pragma unroll
-    for (int r = 0; r < RMAX; r++) {
-      const int rowi = part * R + r;
-      if (r < R && rowi < dk) {
-        S[r] *= g;
-        dot += S[r] * kl[rowi];
-      }
-    }
-    dot = part_sum(dot, JW);
-    const float u = beta * (v_cur - dot);
-    float o = 0.f;
+    for (int u = 0; u < DEPTH; u++) {
+      const int t = t0 + u;
+      if (t >= end) break;
+      float* kl = lds + (u & 1) * 2 * dk;
+      float* ql = kl + dk;
 #pragma unroll
-    for (int r = 0; r < RMAX; r++) {
-      const int rowi = part * R + r;
-      if (r < R && rowi < dk) {
-        S[r] += kl[rowi] * u;
-        o += S[r] * ql[rowi];
+      for (int e = 0; e < PE; e++) {
+        const int i = threadIdx.x + e * blockDim.x;
+        if (i < dk) {
+          kl[i] = pre[u].k[e];
+          ql[i] = pre[u].q[e];
+        }
       }
+      const float beta = sigmoid_f(pre[u].braw);
+      const float g = expf(a_neg * softplus_f(pre[u].araw + dtb));
+      const float v_cur = pre[u].vj;
+      __syncthreads();
+      if (t + DEPTH < end) fetch(pre[u], t + DEPTH);
+      float dot = 0.f;
+#pragma unroll
+      for (int r = 0; r < RMAX; r++) {
+        const int rowi = part * R + r;
+        if (r < R && rowi < dk) {
+          S[r] *= g;
+          dot += S[r] * kl[rowi];
+        }
+      }
+      dot = part_sum(dot, JW);
+      const float uu = beta * (v_cur - dot);
+      float o = 0.f;
+#pragma unroll
+      for (int r = 0; r < RMAX; r++) {
+        const int rowi = part * R + r;
+        if (r < R && rowi < dk) {
+          S[r] += kl[rowi] * uu;
+          o += S[r] * ql[rowi];
+        }
+      }
+      o = part_sum(o, JW);
+      if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = o;
     }
-    o = part_sum(o, JW);
-    if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = o;
   }
   STORE_STATE(S, sbase)
 }
@@ -174,8 +185,8 @@ __global__ void unit_heads_kernel(float* __restrict__ qkv, int Cc, int G,
 // ---------------------------------------------------------------------------
 // RWKV-style time mixing. Per token, with w = exp(-exp(wraw + w0)):
 // o = (S + diag(u) k v^T)^T r; S <- diag(w) S + k v^T.
-template <typename T>
-__global__ void rwkv_kernel(
+template <typename T, int PE>
+__global__ __launch_bounds__(512) void rwkv_kernel(
     float* __restrict__ out,       // [T, H, d]
     const T* __restrict__ r_, const T* __restrict__ k_,
     const T* __restrict__ v_,      // [T, H*d] each
@@ -204,54 +215,63 @@ __global__ void rwkv_kernel(
     const int rowi = part * R + r;
     U[r] = (r < R && rowi < dk) ? u[hh * dk + rowi] : 0.f;
   }
-  float w0r[PEMAX];
+  float w0r[PE];
 #pragma unroll
-  for (int e = 0; e < PEMAX; e++) {
+  for (int e = 0; e < PE; e++) {
     const int i = threadIdx.x + e * blockDim.x;
     w0r[e] = i < dk ? w0[hh * dk + i] : 0.f;
   }
   const int HD = H * dk;
-  float rpre[PEMAX], kpre[PEMAX], wpre[PEMAX], vj;
-  auto fetch = [&](int t) {
+  struct In { float r[PE], k[PE], w[PE], vj; };
+  In pre[DEPTH];
+  const int end = start + len;
+  auto fetch = [&](In& in, int t) {
     const int64_t base = (int64_t)t * HD + hh * dk;
 #pragma unroll
-    for (int e = 0; e < PEMAX; e++) {
+    for (int e = 0; e < PE; e++) {
       const int i = threadIdx.x + e * blockDim.x;
-      rpre[e] = i < dk ? to_f(r_[base + i]) : 0.f;
-      kpre[e] = i < dk ? to_f(k_[base + i]) : 0.f;
-      wpre[e] = i < dk ? to_f(wraw[base + i]) : 0.f;
+      in.r[e] = i < dk ? to_f(r_[base + i]) : 0.f;
+      in.k[e] = i < dk ? to_f(k_[base + i]) : 0.f;
+      in.w[e] = i < dk ? to_f(wraw[base + i]) : 0.f;
     }
-    vj = valid ? to_f(v_[(int64_t)t * H * dv + hh * dv + j]) : 0.f;
+    in.vj = valid ? to_f(v_[(int64_t)t * H * dv + hh * dv + j]) : 0.f;
   };
-  fetch(start);
-  for (int t = start; t < start + len; t++) {
-    float* rl = lds + ((t - start) & 1) * 3 * dk;
-    float* kl = rl + dk;
-    float* wl = rl + 2 * dk;
 #pragma unroll
-    for (int e = 0; e < PEMAX; e++) {
-      const int i = threadIdx.x + e * blockDim.x;
-      if (i < dk) {
-        rl[i] = rpre[e];
-        kl[i] = kpre[e];
-        wl[i] = expf(-expf(wpre[e] + w0r[e]));
-      }
-    }
-    const float v_cur = vj;
-    __syncthreads();
-    if (t + 1 < start + len) fetch(t + 1);
-    float o = 0.f;
+  for (int u = 0; u < DEPTH; u++)
+    if (start + u < end) fetch(pre[u], start + u);
+  for (int t0 = start; t0 < end; t0 += DEPTH) {
 #pragma unroll
-    for (int r = 0; r < RMAX; r++) {
-      const int rowi = part * R + r;
-      if (r < R && rowi < dk) {
-        const float kv = kl[rowi] * v_cur;
-        o += rl[rowi] * (S[r] + U[r] * kv);
-        S[r] = wl[rowi] * S[r] + kv;
+    for (int u = 0; u < DEPTH; u++) {
+      const int t = t0 + u;
+      if (t >= end) break;
+      float* rl = lds + (u & 1) * 3 * dk;
+      float* kl = rl + dk;
+      float* wl = rl + 2 * dk;
+#pragma unroll
+      for (int e = 0; e < PE; e++) {
+        const int i = threadIdx.x + e * blockDim.x;
+        if (i < dk) {
+          rl[i] = pre[u].r[e];
+          kl[i] = pre[u].k[e];
+          wl[i] = expf(-expf(pre[u].w[e] + w0r[e]));
+        }
       }
+      const float v_cur = pre[u].vj;
+      __syncthreads();
+      if (t + DEPTH < end) fetch(pre[u], t + DEPTH);
+      float o = 0.f;
+#pragma unroll
+      for (int r = 0; r < RMAX; r++) {
+        const int rowi = part * R + r;
+        if (r < R && rowi < dk) {
+          const float kv = kl[rowi] * v_cur;
+          o += rl[rowi] * (S[r] + U[r] * kv);
+          S[r] = wl[rowi] * S[r] + kv;
+        }
+      }
+      o = part_sum(o, JW);
+      if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = o;
     }
-    o = part_sum(o, JW);
-    if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = o;
   }
   STORE_STATE(S, sbase)
 }
@@ -261,8 +281,8 @@ __global__ void rwkv_kernel(
 // i = cap tanh((iraw + ib) / cap); f = logsigmoid(cap tanh((fraw + fb) / cap))
 // m' = max(f + m, i); S <- e^(f+m-m') S + e^(i-m') k v^T; n likewise with k;
 // o = S^T q / (max(|n . q|, e^(-m')) + den_eps).
-template <typename T>
-__global__ void mlstm_kernel(
+template <typename T, int PE>
+__global__ __launch_bounds__(512) void mlstm_kernel(
     float* __restrict__ out,  // [T, H, dv]
     const T* __restrict__ proj, int proj_stride, int off_q, int off_k,
     int off_v, int off_i, int off_f, const float* __restrict__ i_bias,
@@ -297,55 +317,64 @@ __global__ void mlstm_kernel(
   float m = fresh ? 0.f : state_m[slot * H + hh];
   const float ib = i_bias[hh], fb = f_bias[hh];
 
-  float kpre[PEMAX], qpre[PEMAX], iraw, fraw, vj;
-  auto fetch = [&](int t) {
+  struct In { float k[PE], q[PE], iraw, fraw, vj; };
+  In pre[DEPTH];
+  const int end = start + len;
+  auto fetch = [&](In& in, int t) {
     const T* row = proj + (int64_t)t * proj_stride;
 #pragma unroll
-    for (int e = 0; e < PEMAX; e++) {
+    for (int e = 0; e < PE; e++) {
       const int i = threadIdx.x + e * blockDim.x;
-      kpre[e] = i < dk ? to_f(row[off_k + hh * dk + i]) : 0.f;
-      qpre[e] = i < dk ? to_f(row[off_q + hh * dk + i]) * qscale : 0.f;
+      in.k[e] = i < dk ? to_f(row[off_k + hh * dk + i]) : 0.f;
+      in.q[e] = i < dk ? to_f(row[off_q + hh * dk + i]) * qscale : 0.f;
     }
-    iraw = to_f(row[off_i + hh]);
-    fraw = to_f(row[off_f + hh]);
-    vj = valid ? to_f(row[off_v + hh * dv + j]) : 0.f;
+    in.iraw = to_f(row[off_i + hh]);
+    in.fraw = to_f(row[off_f + hh]);
+    in.vj = valid ? to_f(row[off_v + hh * dv + j]) : 0.f;
   };
-  fetch(start);
-  for (int t = start; t < start + len; t++) {
-    float* kl = lds + ((t - start) & 1) * 2 * dk;
-    float* ql = kl + dk;
 #pragma unroll
-    for (int e = 0; e < PEMAX; e++) {
-      const int i = threadIdx.x + e * blockDim.x;
-      if (i < dk) {
-        kl[i] = kpre[e];
-        ql[i] = qpre[e];
-      }
-    }
-    const float ig = cap * tanhf((iraw + ib) / cap);
-    const float fg = logsigmoid_f(cap * tanhf((fraw + fb) / cap));
-    const float v_cur = vj;
-    __syncthreads();
-    if (t + 1 < start + len) fetch(t + 1);
-    const float mn = fmaxf(fg + m, ig);
-    const float a = expf(fg + m - mn), b = expf(ig - mn);
-    m = mn;
-    float num = 0.f, nq = 0.f;
+  for (int u = 0; u < DEPTH; u++)
+    if (start + u < end) fetch(pre[u], start + u);
+  for (int t0 = start; t0 < end; t0 += DEPTH) {
 #pragma unroll
-    for (int r = 0; r < RMAX; r++) {
-      const int rowi = part * R + r;
-      if (r < R && rowi < dk) {
-        const float bk = b * kl[rowi];
-        S[r] = a * S[r] + bk * v_cur;
-        N[r] = a * N[r] + bk;
-        num += S[r] * ql[rowi];
-        nq += N[r] * ql[rowi];
+    for (int u = 0; u < DEPTH; u++) {
+      const int t = t0 + u;
+      if (t >= end) break;
+      float* kl = lds + (u & 1) * 2 * dk;
+      float* ql = kl + dk;
+#pragma unroll
+      for (int e = 0; e < PE; e++) {
+        const int i = threadIdx.x + e * blockDim.x;
+        if (i < dk) {
+          kl[i] = pre[u].k[e];
+          ql[i] = pre[u].q[e];
+        }
       }
+      const float ig = cap * tanhf((pre[u].iraw + ib) / cap);
+      const float fg = logsigmoid_f(cap * tanhf((pre[u].fraw + fb) / cap));
+      const float v_cur = pre[u].vj;
+      __syncthreads();
+      if (t + DEPTH < end) fetch(pre[u], t + DEPTH);
+      const float mn = fmaxf(fg + m, ig);
+      const float a = expf(fg + m - mn), b = expf(ig - mn);
+      m = mn;
+      float num = 0.f, nq = 0.f;
+#pragma unroll
+      for (int r = 0; r < RMAX; r++) {
+        const int rowi = part * R + r;
+        if (r < R && rowi < dk) {
+          const float bk = b * kl[rowi];
+          S[r] = a * S[r] + bk * v_cur;
+          N[r] = a * N[r] + bk;
+          num += S[r] * ql[rowi];
+          nq += N[r] * ql[rowi];
+        }
+      }
+      num = part_sum(num, JW);
+      nq = part_sum(nq, JW);
+      const float den = fmaxf(fabsf(nq), expf(-m)) + den_eps;
+      if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = num / den;
     }
-    num = part_sum(num, JW);
-    nq = part_sum(nq, JW);
-    const float den = fmaxf(fabsf(nq), expf(-m)) + den_eps;
-    if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = num / den;
   }
   STORE_STATE(S, sbase)
 }
@@ -433,7 +462,8 @@ void gated_delta_rule(torch::Tensor out, torch::Tensor qkv, torch::Tensor proj,
                      cur_stream(), ptr<float>(qkv), (int)qkv.size(1), (int)G,
                      dk, (float)qscale, (float)unit_eps);
   DISPATCH_ACT(proj, hipLaunchKernelGGL(
-      gated_delta_kernel<T>, dim3(B, H, g.tiles), dim3(g.NW * 64),
+      (dk <= g.NW * 64 ? gated_delta_kernel<T, 1> : gated_delta_kernel<T, PEMAX>),
+      dim3(B, H, g.tiles), dim3(g.NW * 64),
       4 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<float>(qkv),
       cptr<T>(proj), (int)proj.stride(0), (int)off_b, (int)off_a,
       cptr<float>(A_log), cptr<float>(dt_bias), ptr<float>(state), sa, H,
@@ -463,7 +493,8 @@ void rwkv_time_mix(torch::Tensor out, torch::Tensor r, torch::Tensor k,
   SeqArgs sa = seq_args(seq_start, seq_len, seq_slot, seq_pos0, state.size(0));
   Geometry g = geometry(dk, dv);
   DISPATCH_ACT(r, hipLaunchKernelGGL(
-      rwkv_kernel<T>, dim3(B, H, g.tiles), dim3(g.NW * 64),
+      (dk <= g.NW * 64 ? rwkv_kernel<T, 1> : rwkv_kernel<T, PEMAX>),
+      dim3(B, H, g.tiles), dim3(g.NW * 64),
       6 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(r),
       cptr<T>(k), cptr<T>(v), cptr<T>(wraw), cptr<float>(w0), cptr<float>(u),
       ptr<float>(state), sa, H, dk, dv, g.KP, g.R););
@@ -500,7 +531,8 @@ void mlstm_memory(torch::Tensor out, torch::Tensor proj, int64_t off_q,
   SeqArgs sa = seq_args(seq_start, seq_len, seq_slot, seq_pos0, state_S.size(0));
   Geometry g = geometry(dk, dv);
   DISPATCH_ACT(proj, hipLaunchKernelGGL(
-      mlstm_kernel<T>, dim3(B, H, g.tiles), dim3(g.NW * 64),
+      (dk <= g.NW * 64 ? mlstm_kernel<T, 1> : mlstm_kernel<T, PEMAX>),
+      dim3(B, H, g.tiles), dim3(g.NW * 64),
       4 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(proj),
       (int)proj.stride(0), (int)off_q, (int)off_k, (int)off_v, (int)off_i,
       (int)off_f, cptr<float>(i_bias), cptr<float>(f_bias),
