@@ -74,9 +74,12 @@ template <> struct Vec16<bf16_t> {
 // partial dots, 16 keys a pass, 4 passes a chunk; no transposed staging is
 // needed. For the weighted sum a lane owns pairs of adjacent value channels
 // and reads value rows as they lie in the page, eight rows in flight.
-// VEC is off when a key row is not a whole number of 16-byte pieces; EVT
-// is the number of value channels a lane owns.
-template <typename T, int GS, bool VEC, int EVT>
+// FAST needs key rows that are whole 16-byte pieces, an even value size
+// and a page size that is a multiple of 16: then every load address is
+// clamped into range instead of tested, so the loads of a pass issue back
+// to back. Otherwise a plain scalar path runs. EVT is the number of value
+// channels a lane owns.
+template <typename T, int GS, bool FAST, int EVT>
 __global__ __launch_bounds__(1024) void biased_attention_kernel(
     T* __restrict__ out,  // [T, H, dv]
     const T* __restrict__ proj, int proj_stride, int off_q,
@@ -113,12 +116,10 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
     b2[a] = has_bias ? r2[h0 + a] : 0.f;
   }
   const int quad = lane >> 2, qq = lane & 3;
-  const int nvec = dk / VN;        // used when VEC
-  const bool run16 = ps % 16 == 0;  // a 16-key pass lies in one page
-  // adjacent channels load as one word when rows stay aligned
-  const bool pair = (dv & 1) == 0 &&
-                    reinterpret_cast<uintptr_t>(vcache) % 8 == 0;
+  const int nvec = dk / VN;  // 16-byte pieces of a key row (FAST)
 
+  // l is kept per lane (the sum over the keys this lane scored, each key
+  // counted by the 4 lanes of its quad) and only reduced at the end
   float m[GS], l[GS], acc[GS][EVT];
 #pragma unroll
   for (int a = 0; a < GS; a++) {
@@ -136,44 +137,43 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
 #pragma unroll
     for (int p = 0; p < 4; p++) {
       const int j = j0 + 16 * p + quad;
+      const int jc = min(j, ctx - 1);  // loads stay in range, masked below
       float d[GS];
 #pragma unroll
       for (int a = 0; a < GS; a++) d[a] = 0.f;
-      if (j < ctx) {
-        const int64_t page = table[j / ps];
-        const T* k = kcache + ((page * G + g) * ps + (j % ps)) * dk;
-        if (VEC) {
-          for (int v0 = qq; v0 < nvec; v0 += 16) {
-            Vec16<T> kv[4];
+      const int64_t page = table[jc / ps];
+      const T* k = kcache + ((page * G + g) * ps + (jc % ps)) * dk;
+      if (FAST) {
+        for (int v0 = qq; v0 < nvec; v0 += 16) {
+          Vec16<T> kv[4];
 #pragma unroll
-            for (int u = 0; u < 4; u++)
-              if (v0 + 4 * u < nvec)
-                kv[u].v = *reinterpret_cast<const decltype(kv[u].v)*>(
-                    k + (v0 + 4 * u) * VN);
+          for (int u = 0; u < 4; u++)
+            kv[u].v = *reinterpret_cast<const decltype(kv[u].v)*>(
+                k + min(v0 + 4 * u, nvec - 1) * VN);
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-              const int v = v0 + 4 * u;
-              if (v < nvec) {
+          for (int u = 0; u < 4; u++) {
+            const int v = min(v0 + 4 * u, nvec - 1);
+            const float on = v0 + 4 * u < nvec ? 1.f : 0.f;
 #pragma unroll
-                for (int a = 0; a < GS; a++) {
-                  const float4* q4 =
-                      reinterpret_cast<const float4*>(qs + a * dk + v * VN);
+            for (int a = 0; a < GS; a++) {
+              const float4* q4 =
+                  reinterpret_cast<const float4*>(qs + a * dk + v * VN);
+              float part = 0.f;
 #pragma unroll
-                  for (int i4 = 0; i4 < VN / 4; i4++) {
-                    const float4 q = q4[i4];
-                    d[a] += q.x * kv[u].get(4 * i4) + q.y * kv[u].get(4 * i4 + 1) +
-                            q.z * kv[u].get(4 * i4 + 2) + q.w * kv[u].get(4 * i4 + 3);
-                  }
-                }
+              for (int i4 = 0; i4 < VN / 4; i4++) {
+                const float4 q = q4[i4];
+                part += q.x * kv[u].get(4 * i4) + q.y * kv[u].get(4 * i4 + 1) +
+                        q.z * kv[u].get(4 * i4 + 2) + q.w * kv[u].get(4 * i4 + 3);
               }
+              d[a] += on * part;
             }
           }
-        } else {
-          for (int i = qq; i < dk; i += 4) {
-            const float kf = to_f(k[i]);
+        }
+      } else {
+        for (int i = qq; i < dk; i += 4) {
+          const float kf = to_f(k[i]);
 #pragma unroll
-            for (int a = 0; a < GS; a++) d[a] += qs[a * dk + i] * kf;
-          }
+          for (int a = 0; a < GS; a++) d[a] += qs[a * dk + i] * kf;
         }
       }
 #pragma unroll
@@ -181,12 +181,8 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
         float x = d[a];
         x += __shfl_xor(x, 1, 64);
         x += __shfl_xor(x, 2, 64);
-        if (j < ctx) {
-          if (has_bias) x -= b1[a] * log1pf(b2[a] * (float)(pos - j));
-        } else {
-          x = -INFINITY;
-        }
-        sc[p][a] = x;
+        if (has_bias) x -= b1[a] * log1pf(b2[a] * (float)(pos - jc));
+        sc[p][a] = j < ctx ? x : -INFINITY;
       }
     }
     // ---- online softmax (every lane of a quad holds the same score) ----
@@ -202,7 +198,7 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
         pr[p][a] = expf(sc[p][a] - mx);  // 0 for masked keys
         sum += pr[p][a];
       }
-      l[a] = l[a] * corr + 0.25f * wave_sum(sum);  // 4 lanes per key
+      l[a] = l[a] * corr + sum;
       m[a] = mx;
 #pragma unroll
       for (int e = 0; e < EVT; e++) acc[a][e] *= corr;
@@ -214,66 +210,68 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
       const int jp = j0 + 16 * p;
       const int nk = min(16, ctx - jp);
       if (nk <= 0) break;
-      const T* vrun = nullptr;
-      if (run16)
-        vrun = vcache + (((int64_t)table[jp / ps] * G + g) * ps + (jp % ps)) * dv;
-      for (int k0 = 0; k0 < nk; k0 += 8) {
-        float vf[8][EVT];
+      if (FAST) {
+        // the 16 keys of a pass lie in one page; rows past the context
+        // are read from the last valid row and weigh 0
+        const T* vrun =
+            vcache + (((int64_t)table[jp / ps] * G + g) * ps + (jp % ps)) * dv;
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-          const int kk = k0 + u;
-          if (kk < nk) {
-            const T* v;
-            if (run16) {
-              v = vrun + (int64_t)kk * dv;
-            } else {
-              const int j = jp + kk;
-              v = vcache + (((int64_t)table[j / ps] * G + g) * ps + (j % ps)) * dv;
-            }
+        for (int k0 = 0; k0 < 16; k0 += 8) {
+          if (k0 >= nk) break;
+          float vf[8][EVT];
+#pragma unroll
+          for (int u = 0; u < 8; u++) {
+            const T* v = vrun + (int64_t)min(k0 + u, nk - 1) * dv;
 #pragma unroll
             for (int e = 0; e < EVT; e += 2) {
-              const int ch = (e / 2) * 128 + 2 * lane;
-              if (pair) {
-                if (ch < dv) {  // dv even: ch + 1 < dv as well
-                  if (sizeof(T) == 2) {
-                    const uint32_t w = *reinterpret_cast<const uint32_t*>(v + ch);
-                    union { float f; uint32_t u; } c0, c1;
-                    c0.u = w << 16;
-                    c1.u = w & 0xffff0000u;
-                    vf[u][e] = c0.f;
-                    if (e + 1 < EVT) vf[u][e + 1] = c1.f;
-                  } else {
-                    const float2 w = *reinterpret_cast<const float2*>(v + ch);
-                    vf[u][e] = w.x;
-                    if (e + 1 < EVT) vf[u][e + 1] = w.y;
-                  }
-                } else {
-                  vf[u][e] = 0.f;
-                  if (e + 1 < EVT) vf[u][e + 1] = 0.f;
-                }
+              const int ch = min((e / 2) * 128 + 2 * lane, dv - 2);
+              if (sizeof(T) == 2) {
+                const uint32_t w = *reinterpret_cast<const uint32_t*>(v + ch);
+                union { float f; uint32_t u; } c0, c1;
+                c0.u = w << 16;
+                c1.u = w & 0xffff0000u;
+                vf[u][e] = c0.f;
+                vf[u][e + 1] = c1.f;
               } else {
-                vf[u][e] = ch < dv ? to_f(v[ch]) : 0.f;
-                if (e + 1 < EVT) vf[u][e + 1] = ch + 1 < dv ? to_f(v[ch + 1]) : 0.f;
+                const float2 w = *reinterpret_cast<const float2*>(v + ch);
+                vf[u][e] = w.x;
+                vf[u][e + 1] = w.y;
               }
             }
-          } else {
+          }
 #pragma unroll
-            for (int e = 0; e < EVT; e++) vf[u][e] = 0.f;
+          for (int u = 0; u < 8; u++) {
+#pragma unroll
+            for (int a = 0; a < GS; a++) {
+              const float w = __shfl(pr[p][a], (k0 + u) << 2, 64);
+#pragma unroll
+              for (int e = 0; e < EVT; e++) acc[a][e] += w * vf[u][e];
+            }
           }
         }
+      } else {
+        for (int kk = 0; kk < nk; kk++) {
+          const int j = jp + kk;
+          const T* v =
+              vcache + (((int64_t)table[j / ps] * G + g) * ps + (j % ps)) * dv;
+          float w[GS];
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-          const int src = ((k0 + u) & 15) << 2;  // lane that holds this key
+          for (int a = 0; a < GS; a++) w[a] = __shfl(pr[p][a], kk << 2, 64);
 #pragma unroll
-          for (int a = 0; a < GS; a++) {
-            const float w = __shfl(pr[p][a], src, 64);
+          for (int e = 0; e < EVT; e++) {
+            const int ch = (e / 2) * 128 + 2 * lane + (e & 1);
+            if (ch < dv) {
+              const float vf = to_f(v[ch]);
 #pragma unroll
-            for (int e = 0; e < EVT; e++) acc[a][e] += w * vf[u][e];
+              for (int a = 0; a < GS; a++) acc[a][e] += w[a] * vf;
+            }
           }
         }
       }
     }
   }
+#pragma unroll
+  for (int a = 0; a < GS; a++) l[a] = 0.25f * wave_sum(l[a]);
   // ---- merge the waves ----
   const int MS = 2 + dv;  // floats per (wave, head) record
 #pragma unroll
@@ -327,8 +325,9 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
   const size_t lds = (size_t)(GS * dk + NW * GS * (2 + dv)) * sizeof(float);
   TORCH_CHECK(lds <= 64 * 1024,
               "seqmix: attention head sizes exceed the LDS budget");
-  const bool vec = (dk * sizeof(T)) % 16 == 0 &&
-                   reinterpret_cast<uintptr_t>(kcache.data_ptr()) % 16 == 0;
+  const bool vec = (dk * sizeof(T)) % 16 == 0 && dv % 2 == 0 && ps % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(kcache.data_ptr()) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(vcache.data_ptr()) % 8 == 0;
   const bool small = dv <= 128;
 #define LAUNCH_ATT(GS_, VEC_, EVT_)                                         \
   hipLaunchKernelGGL((biased_attention_kernel<T, GS_, VEC_, EVT_>),         \

@@ -5,9 +5,12 @@
 //
 // All three recurrences are independent per value column j: column j of S
 // is only ever combined with the token's key-side vectors. A thread keeps
-// R rows of one column in registers; KP threads (adjacent at lane distance
-// JW = 64 / KP) share a column and reduce their partial dot products with
-// lane shuffles. R <= RMAX and KP is a power of two, so dk <= RMAX * 64.
+// RT rows (16 or 32, a template constant) of one column in registers; KP
+// threads (adjacent at lane distance JW = 64 / KP) share a column and
+// reduce their partial dot products with lane shuffles. KP is a power of
+// two, so dk <= 32 * 64. Rows past dk are zero padding: they are staged as
+// zeros and stay zero, which keeps the per-token loops free of bounds
+// tests (fixed trip counts, 16-byte LDS reads issued back to back).
 // State is fp32 in HBM, loaded once per step and stored once.
 //
 // The walk over a portion is latency bound (one token depends on the one
@@ -21,7 +24,6 @@
 
 namespace {
 
-constexpr int RMAX = 32;
 constexpr int PEMAX = 4;  // staged elements per thread and vector
 constexpr int DEPTH = 4;  // tokens fetched ahead
 
@@ -33,20 +35,21 @@ struct SeqArgs {
 };
 
 struct Geometry {
-  int KP, R, JW, NW, tiles;
+  int KP, RT, DKP, JW, NW, tiles;
 };
 
 inline Geometry geometry(int dk, int dv) {
   Geometry g;
   g.KP = 1;
-  while (g.KP * RMAX < dk) g.KP <<= 1;
+  while (g.KP * 32 < dk) g.KP <<= 1;
   TORCH_CHECK(g.KP <= 64, "seqmix: key size too large for the recurrence");
-  g.R = (dk + g.KP - 1) / g.KP;
+  g.RT = (dk + g.KP - 1) / g.KP <= 16 ? 16 : 32;
+  g.DKP = g.KP * g.RT;  // padded key size
   g.JW = 64 / g.KP;
   const int waves = (dv + g.JW - 1) / g.JW;
   g.NW = waves < 4 ? waves : 4;
   // enough threads to stage a key-side vector with PEMAX elements each
-  const int need = (dk + 64 * PEMAX - 1) / (64 * PEMAX);
+  const int need = (g.DKP + 64 * PEMAX - 1) / (64 * PEMAX);
   if (g.NW < need) g.NW = need;
   g.tiles = (waves + g.NW - 1) / g.NW;
   return g;
@@ -59,22 +62,29 @@ DEVINL float part_sum(float x, int JW) {
 }
 
 #define LOAD_STATE(S, base, fresh)                                    \
-  _Pragma("unroll") for (int r = 0; r < RMAX; r++) {                   \
-    const int row = part * R + r;                                      \
-    S[r] = (!fresh && r < R && row < dk && valid)                      \
-               ? base[(int64_t)row * dv + j] : 0.f;                    \
+  _Pragma("unroll") for (int r = 0; r < RT; r++) {                     \
+    const int row = part * RT + r;                                     \
+    S[r] = (!fresh && row < dk && valid) ? base[(int64_t)row * dv + j] \
+                                         : 0.f;                        \
   }
 #define STORE_STATE(S, base)                                          \
-  _Pragma("unroll") for (int r = 0; r < RMAX; r++) {                   \
-    const int row = part * R + r;                                      \
-    if (r < R && row < dk && valid) base[(int64_t)row * dv + j] = S[r]; \
+  _Pragma("unroll") for (int r = 0; r < RT; r++) {                     \
+    const int row = part * RT + r;                                     \
+    if (row < dk && valid) base[(int64_t)row * dv + j] = S[r];         \
+  }
+// RT staged values of this thread's rows, as 16-byte LDS reads
+#define READ_ROWS(dst, vec)                                           \
+  _Pragma("unroll") for (int r4 = 0; r4 < RT / 4; r4++) {              \
+    const float4 x = reinterpret_cast<const float4*>(vec + part * RT)[r4]; \
+    dst[4 * r4] = x.x; dst[4 * r4 + 1] = x.y;                          \
+    dst[4 * r4 + 2] = x.z; dst[4 * r4 + 3] = x.w;                      \
   }
 
 // ---------------------------------------------------------------------------
 // Gated delta rule. Per token: S <- g S; u = beta (v - S^T k);
 // S <- S + k u^T; o = S^T q. q and k arrive after the short convolution and
 // are made unit vectors here (q also scaled by qscale).
-template <typename T, int PE>
+template <typename T, int PE, int RT>
 __global__ __launch_bounds__(512) void gated_delta_kernel(
     float* __restrict__ out,          // [T, H, dv]
     const float* __restrict__ qkv,    // [T, Cq + Ck + Cv]: unit k, scaled
@@ -82,8 +92,10 @@ __global__ __launch_bounds__(512) void gated_delta_kernel(
     const T* __restrict__ proj, int proj_stride, int off_b, int off_a,
     const float* __restrict__ A_log, const float* __restrict__ dt_bias,
     float* __restrict__ state,        // [slots, H, dk, dv]
-    SeqArgs sa, int H, int G, int dk, int dv, int KP, int R) {
-  extern __shared__ float lds[];  // [2 buffers][k | q][dk]
+    SeqArgs sa, int H, int G, int dk, int dv, int KP) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  // [2 buffers][k | q][DKP]
+  const int DKP = KP * RT;
   const int s = blockIdx.x, hh = blockIdx.y;
   const int len = sa.seq_len[s];
   if (len == 0) return;
@@ -98,7 +110,7 @@ __global__ __launch_bounds__(512) void gated_delta_kernel(
   const int kvh = hh / (H / G);
   const int Cq = G * dk, Cc = 2 * G * dk + H * dv;
   float* sbase = state + ((int64_t)sa.seq_slot[s] * H + hh) * dk * dv;
-  float S[RMAX];
+  float S[RT];
   LOAD_STATE(S, sbase, fresh)
   const float a_neg = -expf(A_log[hh]);
   const float dtb = dt_bias[hh];
@@ -126,12 +138,12 @@ __global__ __launch_bounds__(512) void gated_delta_kernel(
     for (int u = 0; u < DEPTH; u++) {
       const int t = t0 + u;
       if (t >= end) break;
-      float* kl = lds + (u & 1) * 2 * dk;
-      float* ql = kl + dk;
+      float* kl = lds + (u & 1) * 2 * DKP;
+      float* ql = kl + DKP;
 #pragma unroll
       for (int e = 0; e < PE; e++) {
         const int i = threadIdx.x + e * blockDim.x;
-        if (i < dk) {
+        if (i < DKP) {
           kl[i] = pre[u].k[e];
           ql[i] = pre[u].q[e];
         }
@@ -141,25 +153,22 @@ __global__ __launch_bounds__(512) void gated_delta_kernel(
       const float v_cur = pre[u].vj;
       __syncthreads();
       if (t + DEPTH < end) fetch(pre[u], t + DEPTH);
+      float kr[RT], qr[RT];
+      READ_ROWS(kr, kl)
+      READ_ROWS(qr, ql)
       float dot = 0.f;
 #pragma unroll
-      for (int r = 0; r < RMAX; r++) {
-        const int rowi = part * R + r;
-        if (r < R && rowi < dk) {
-          S[r] *= g;
-          dot += S[r] * kl[rowi];
-        }
+      for (int r = 0; r < RT; r++) {
+        S[r] *= g;
+        dot += S[r] * kr[r];
       }
       dot = part_sum(dot, JW);
       const float uu = beta * (v_cur - dot);
       float o = 0.f;
 #pragma unroll
-      for (int r = 0; r < RMAX; r++) {
-        const int rowi = part * R + r;
-        if (r < R && rowi < dk) {
-          S[r] += kl[rowi] * uu;
-          o += S[r] * ql[rowi];
-        }
+      for (int r = 0; r < RT; r++) {
+        S[r] += kr[r] * uu;
+        o += S[r] * qr[r];
       }
       o = part_sum(o, JW);
       if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = o;
@@ -185,7 +194,7 @@ __global__ void unit_heads_kernel(float* __restrict__ qkv, int Cc, int G,
 // ---------------------------------------------------------------------------
 // RWKV-style time mixing. Per token, with w = exp(-exp(wraw + w0)):
 // o = (S + diag(u) k v^T)^T r; S <- diag(w) S + k v^T.
-template <typename T, int PE>
+template <typename T, int PE, int RT>
 __global__ __launch_bounds__(512) void rwkv_kernel(
     float* __restrict__ out,       // [T, H, d]
     const T* __restrict__ r_, const T* __restrict__ k_,
@@ -194,8 +203,10 @@ __global__ __launch_bounds__(512) void rwkv_kernel(
     const float* __restrict__ w0,  // [H*d]
     const float* __restrict__ u,   // [H, d]
     float* __restrict__ state,     // [slots, H, d, d]
-    SeqArgs sa, int H, int dk, int dv, int KP, int R) {
-  extern __shared__ float lds[];  // [2 buffers][r | k | w][dk]
+    SeqArgs sa, int H, int dk, int dv, int KP) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  // [2 buffers][r | k | w][DKP]
+  const int DKP = KP * RT;
   const int s = blockIdx.x, hh = blockIdx.y;
   const int len = sa.seq_len[s];
   if (len == 0) return;
@@ -208,12 +219,12 @@ __global__ __launch_bounds__(512) void rwkv_kernel(
   const int j = (blockIdx.z * nw + wave) * JW + (lane % JW);
   const bool valid = j < dv;
   float* sbase = state + ((int64_t)sa.seq_slot[s] * H + hh) * dk * dv;
-  float S[RMAX], U[RMAX];
+  float S[RT], U[RT];
   LOAD_STATE(S, sbase, fresh)
 #pragma unroll
-  for (int r = 0; r < RMAX; r++) {
-    const int rowi = part * R + r;
-    U[r] = (r < R && rowi < dk) ? u[hh * dk + rowi] : 0.f;
+  for (int r = 0; r < RT; r++) {
+    const int rowi = part * RT + r;
+    U[r] = rowi < dk ? u[hh * dk + rowi] : 0.f;
   }
   float w0r[PE];
 #pragma unroll
@@ -244,13 +255,13 @@ __global__ __launch_bounds__(512) void rwkv_kernel(
     for (int u = 0; u < DEPTH; u++) {
       const int t = t0 + u;
       if (t >= end) break;
-      float* rl = lds + (u & 1) * 3 * dk;
-      float* kl = rl + dk;
-      float* wl = rl + 2 * dk;
+      float* rl = lds + (u & 1) * 3 * DKP;
+      float* kl = rl + DKP;
+      float* wl = rl + 2 * DKP;
 #pragma unroll
       for (int e = 0; e < PE; e++) {
         const int i = threadIdx.x + e * blockDim.x;
-        if (i < dk) {
+        if (i < DKP) {
           rl[i] = pre[u].r[e];
           kl[i] = pre[u].k[e];
           wl[i] = expf(-expf(pre[u].w[e] + w0r[e]));
@@ -259,15 +270,16 @@ __global__ __launch_bounds__(512) void rwkv_kernel(
       const float v_cur = pre[u].vj;
       __syncthreads();
       if (t + DEPTH < end) fetch(pre[u], t + DEPTH);
+      float rr[RT], kr[RT], wr[RT];
+      READ_ROWS(rr, rl)
+      READ_ROWS(kr, kl)
+      READ_ROWS(wr, wl)
       float o = 0.f;
 #pragma unroll
-      for (int r = 0; r < RMAX; r++) {
-        const int rowi = part * R + r;
-        if (r < R && rowi < dk) {
-          const float kv = kl[rowi] * v_cur;
-          o += rl[rowi] * (S[r] + U[r] * kv);
-          S[r] = wl[rowi] * S[r] + kv;
-        }
+      for (int r = 0; r < RT; r++) {
+        const float kv = kr[r] * v_cur;
+        o += rr[r] * (S[r] + U[r] * kv);
+        S[r] = wr[r] * S[r] + kv;
       }
       o = part_sum(o, JW);
       if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = o;
@@ -281,7 +293,7 @@ __global__ __launch_bounds__(512) void rwkv_kernel(
 // i = cap tanh((iraw + ib) / cap); f = logsigmoid(cap tanh((fraw + fb) / cap))
 // m' = max(f + m, i); S <- e^(f+m-m') S + e^(i-m') k v^T; n likewise with k;
 // o = S^T q / (max(|n . q|, e^(-m')) + den_eps).
-template <typename T, int PE>
+template <typename T, int PE, int RT>
 __global__ __launch_bounds__(512) void mlstm_kernel(
     float* __restrict__ out,  // [T, H, dv]
     const T* __restrict__ proj, int proj_stride, int off_q, int off_k,
@@ -290,9 +302,11 @@ __global__ __launch_bounds__(512) void mlstm_kernel(
     float* __restrict__ state_S,        // [slots, H, dk, dv]
     const float* __restrict__ state_n,  // [slots, H, dk]
     const float* __restrict__ state_m,  // [slots, H]
-    SeqArgs sa, int H, int dk, int dv, int KP, int R, float qscale, float cap,
+    SeqArgs sa, int H, int dk, int dv, int KP, float qscale, float cap,
     float den_eps) {
-  extern __shared__ float lds[];  // [2 buffers][k | q][dk]
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  // [2 buffers][k | q][DKP]
+  const int DKP = KP * RT;
   const int s = blockIdx.x, hh = blockIdx.y;
   const int len = sa.seq_len[s];
   if (len == 0) return;
@@ -307,12 +321,12 @@ __global__ __launch_bounds__(512) void mlstm_kernel(
   const int slot = sa.seq_slot[s];
   float* sbase = state_S + ((int64_t)slot * H + hh) * dk * dv;
   const float* nbase = state_n + ((int64_t)slot * H + hh) * dk;
-  float S[RMAX], N[RMAX];
+  float S[RT], N[RT];
   LOAD_STATE(S, sbase, fresh)
 #pragma unroll
-  for (int r = 0; r < RMAX; r++) {
-    const int rowi = part * R + r;
-    N[r] = (!fresh && r < R && rowi < dk) ? nbase[rowi] : 0.f;
+  for (int r = 0; r < RT; r++) {
+    const int rowi = part * RT + r;
+    N[r] = (!fresh && rowi < dk) ? nbase[rowi] : 0.f;
   }
   float m = fresh ? 0.f : state_m[slot * H + hh];
   const float ib = i_bias[hh], fb = f_bias[hh];
@@ -340,12 +354,12 @@ __global__ __launch_bounds__(512) void mlstm_kernel(
     for (int u = 0; u < DEPTH; u++) {
       const int t = t0 + u;
       if (t >= end) break;
-      float* kl = lds + (u & 1) * 2 * dk;
-      float* ql = kl + dk;
+      float* kl = lds + (u & 1) * 2 * DKP;
+      float* ql = kl + DKP;
 #pragma unroll
       for (int e = 0; e < PE; e++) {
         const int i = threadIdx.x + e * blockDim.x;
-        if (i < dk) {
+        if (i < DKP) {
           kl[i] = pre[u].k[e];
           ql[i] = pre[u].q[e];
         }
@@ -358,17 +372,17 @@ __global__ __launch_bounds__(512) void mlstm_kernel(
       const float mn = fmaxf(fg + m, ig);
       const float a = expf(fg + m - mn), b = expf(ig - mn);
       m = mn;
+      float kr[RT], qr[RT];
+      READ_ROWS(kr, kl)
+      READ_ROWS(qr, ql)
       float num = 0.f, nq = 0.f;
 #pragma unroll
-      for (int r = 0; r < RMAX; r++) {
-        const int rowi = part * R + r;
-        if (r < R && rowi < dk) {
-          const float bk = b * kl[rowi];
-          S[r] = a * S[r] + bk * v_cur;
-          N[r] = a * N[r] + bk;
-          num += S[r] * ql[rowi];
-          nq += N[r] * ql[rowi];
-        }
+      for (int r = 0; r < RT; r++) {
+        const float bk = b * kr[r];
+        S[r] = a * S[r] + bk * v_cur;
+        N[r] = a * N[r] + bk;
+        num += S[r] * qr[r];
+        nq += N[r] * qr[r];
       }
       num = part_sum(num, JW);
       nq = part_sum(nq, JW);
@@ -417,6 +431,13 @@ __global__ void mlstm_nm_kernel(
   if (threadIdx.x == 0) state_m[slot * H + hh] = m_end;
 }
 
+// kernel<T, PE, RT> for a geometry: PE = 1 when one pass of the workgroup
+// stages a whole padded key vector
+#define PICK_KERNEL(K, g)                                                    \
+  ((g).DKP <= (g).NW * 64                                                    \
+       ? ((g).RT == 16 ? K<T, 1, 16> : K<T, 1, 32>)                          \
+       : ((g).RT == 16 ? K<T, PEMAX, 16> : K<T, PEMAX, 32>))
+
 SeqArgs seq_args(const torch::Tensor& seq_start, const torch::Tensor& seq_len,
                  const torch::Tensor& seq_slot, const torch::Tensor& seq_pos0,
                  int64_t slots) {
@@ -462,12 +483,11 @@ void gated_delta_rule(torch::Tensor out, torch::Tensor qkv, torch::Tensor proj,
                      cur_stream(), ptr<float>(qkv), (int)qkv.size(1), (int)G,
                      dk, (float)qscale, (float)unit_eps);
   DISPATCH_ACT(proj, hipLaunchKernelGGL(
-      (dk <= g.NW * 64 ? gated_delta_kernel<T, 1> : gated_delta_kernel<T, PEMAX>),
-      dim3(B, H, g.tiles), dim3(g.NW * 64),
-      4 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<float>(qkv),
-      cptr<T>(proj), (int)proj.stride(0), (int)off_b, (int)off_a,
-      cptr<float>(A_log), cptr<float>(dt_bias), ptr<float>(state), sa, H,
-      (int)G, dk, dv, g.KP, g.R););
+      PICK_KERNEL(gated_delta_kernel, g), dim3(B, H, g.tiles),
+      dim3(g.NW * 64), 4 * g.DKP * sizeof(float), cur_stream(),
+      ptr<float>(out), cptr<float>(qkv), cptr<T>(proj), (int)proj.stride(0),
+      (int)off_b, (int)off_a, cptr<float>(A_log), cptr<float>(dt_bias),
+      ptr<float>(state), sa, H, (int)G, dk, dv, g.KP););
 }
 
 void rwkv_time_mix(torch::Tensor out, torch::Tensor r, torch::Tensor k,
@@ -493,11 +513,10 @@ void rwkv_time_mix(torch::Tensor out, torch::Tensor r, torch::Tensor k,
   SeqArgs sa = seq_args(seq_start, seq_len, seq_slot, seq_pos0, state.size(0));
   Geometry g = geometry(dk, dv);
   DISPATCH_ACT(r, hipLaunchKernelGGL(
-      (dk <= g.NW * 64 ? rwkv_kernel<T, 1> : rwkv_kernel<T, PEMAX>),
-      dim3(B, H, g.tiles), dim3(g.NW * 64),
-      6 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(r),
+      PICK_KERNEL(rwkv_kernel, g), dim3(B, H, g.tiles), dim3(g.NW * 64),
+      6 * g.DKP * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(r),
       cptr<T>(k), cptr<T>(v), cptr<T>(wraw), cptr<float>(w0), cptr<float>(u),
-      ptr<float>(state), sa, H, dk, dv, g.KP, g.R););
+      ptr<float>(state), sa, H, dk, dv, g.KP););
 }
 
 void mlstm_memory(torch::Tensor out, torch::Tensor proj, int64_t off_q,
@@ -531,13 +550,12 @@ void mlstm_memory(torch::Tensor out, torch::Tensor proj, int64_t off_q,
   SeqArgs sa = seq_args(seq_start, seq_len, seq_slot, seq_pos0, state_S.size(0));
   Geometry g = geometry(dk, dv);
   DISPATCH_ACT(proj, hipLaunchKernelGGL(
-      (dk <= g.NW * 64 ? mlstm_kernel<T, 1> : mlstm_kernel<T, PEMAX>),
-      dim3(B, H, g.tiles), dim3(g.NW * 64),
-      4 * dk * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(proj),
+      PICK_KERNEL(mlstm_kernel, g), dim3(B, H, g.tiles), dim3(g.NW * 64),
+      4 * g.DKP * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(proj),
       (int)proj.stride(0), (int)off_q, (int)off_k, (int)off_v, (int)off_i,
       (int)off_f, cptr<float>(i_bias), cptr<float>(f_bias),
       ptr<float>(state_S), ptr<float>(state_n), ptr<float>(state_m), sa, H, dk,
-      dv, g.KP, g.R, (float)qscale, (float)cap, (float)den_eps);
+      dv, g.KP, (float)qscale, (float)cap, (float)den_eps);
     hipLaunchKernelGGL(
       mlstm_nm_kernel<T>, dim3(B, H), dim3(dk < 64 ? 64 : (dk > 256 ? 256 : (dk + 63) / 64 * 64)),
       0, cur_stream(), cptr<T>(proj), (int)proj.stride(0), (int)off_k,

@@ -86,13 +86,23 @@ class GraphRunner:
         kv_pool = self.runner.kv_pool
         meta = self._meta(bc)
         torch.cuda.synchronize()
-        # warm up the exact op sequence on a side stream first
+        # warm up the exact op sequence on a side stream first. Recurrent
+        # state is not idempotent (unlike a cache write to the same slot):
+        # the warm-up runs with empty spans so no state advances, and the
+        # replay that follows the capture is the only real execution
+        saved_len = None
+        if self.seq_model:
+            saved_len = self.seq_len[:bc].clone()
+            self.seq_len[:bc].zero_()
         s = torch.cuda.Stream()
         with torch.cuda.stream(s):
             h = model.forward(self.input_ids[:bc], kv_pool, meta)
             self.logits[:bc] = model.compute_logits(h)
         torch.cuda.current_stream().wait_stream(s)
         torch.cuda.synchronize()
+        if saved_len is not None:
+            self.seq_len[:bc].copy_(saved_len)
+            torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g, pool=self._graph_pool):
             h = model.forward(self.input_ids[:bc], kv_pool, meta)

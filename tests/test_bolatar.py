@@ -232,6 +232,54 @@ def test_convolution_widths(tmp_path, device, taps):
         assert U.rel_err(U.replay(eng, "r", toks, sizes), want) < U.TOL["float32"]
 
 
+@pytest.mark.parametrize("device", DEVICES)
+def test_odd_sizes(tmp_path, device):
+    """Sizes that fit no vector width: the scalar paths of the kernels, a
+    group of three query heads per kv head, a key size above 32 rows per
+    lane group and a value size that is not a multiple of the wave."""
+    par = copy.deepcopy(U.PARALLEL)
+    par["mixer"]["left"].update(heads=3, kv_heads=1, dim=10, vdim=7)
+    par["mixer"]["right"].update(heads=2, dim=9)
+    dl = copy.deepcopy(U.DELTA)
+    dl["mixer"].update(heads=2, kv_heads=1, dim=70, vdim=5)
+    ml = copy.deepcopy(U.MLSTM)
+    ml["mixer"].update(heads=3, dim=37, vdim=70)
+    path, cfg, W = _case(tmp_path, [par, dl, ml], seed=13, width=66, vocab=91)
+    toks = U.tokens_for(cfg, 40, 8)
+    want = oracle.forward(cfg, W, toks)
+    eng = U.make_engine(path, device, page_size=8, pages=12)
+    for sizes in ([40], [3, 1, 1, 19, 2]):
+        assert U.rel_err(U.replay(eng, "r", toks, sizes), want) < U.TOL["float32"]
+
+
+@pytest.mark.gpu
+def test_bf16_and_graph_decode(full_ckpt):
+    """bf16 serving path on the GPU: logits close to the oracle, and greedy
+    decoding through captured hipGraphs equals the eager engine token for
+    token (every replay checked against eager work in between)."""
+    from dynamo_amd.engine import SamplingParams
+    path, cfg, W = full_ckpt
+    toks = U.tokens_for(cfg, 70, 50)
+    want = oracle.forward(cfg, W, toks)
+    eng = U.make_engine(path, "cuda:0", dtype="bfloat16")
+    assert U.rel_err(U.replay(eng, "r", toks, [33, 2, 1]), want) < U.TOL["bfloat16"]
+    outs = []
+    for graphs in (False, True):
+        e = U.make_engine(path, "cuda:0", dtype="float32", graphs=graphs,
+                          slots=4)
+        for i in range(3):
+            e.add_request(f"g{i}", U.tokens_for(cfg, 9 + 7 * i, 60 + i),
+                          SamplingParams(max_tokens=20, ignore_eos=True))
+        got = {}
+        while e.has_work():
+            for so in e.step():
+                got.setdefault(so.req_id, []).append(so.new_token)
+        if graphs:
+            assert e.graph_runner is not None and e.graph_runner.graphs
+        outs.append(got)
+    assert outs[0] == outs[1]
+
+
 # -- generation through the engine's own entry point ------------------------
 @pytest.mark.parametrize("device", DEVICES)
 def test_greedy_generation_matches_oracle(full_ckpt, device):
