@@ -319,7 +319,10 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
   const int T_ = out.size(0), H = out.size(1), dv = out.size(2);
   const int G = kcache.size(1), ps = kcache.size(2), dk = kcache.size(3);
   const int gsz = H / G;
-  const int GS = gsz % 4 == 0 ? 4 : (gsz % 2 == 0 ? 2 : 1);
+  // heads of a group share each key/value load; with few rows in flight a
+  // smaller group gives the chip more workgroups instead
+  int GS = gsz % 4 == 0 ? 4 : (gsz % 2 == 0 ? 2 : 1);
+  if (GS == 4 && T_ * (H / 4) < 256) GS = 2;
   // few rows in flight (decoding): 16 waves split the keys of each row
   const int NW = T_ * (H / GS) <= 2048 ? 16 : 4;
   const size_t lds = (size_t)(GS * dk + NW * GS * (2 + dv)) * sizeof(float);
