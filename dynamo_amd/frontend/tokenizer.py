@@ -37,20 +37,52 @@ class ByteTokenizer:
         ids = list(text.encode("utf-8"))
         return ([self.bos_id] if add_bos else []) + ids
 
-    def decode(self, ids: List[int]) -> str:
-        bs = bytes(i for i in ids if 0 <= i < 256)
-        try:
-            return bs.decode("utf-8")
-        except UnicodeDecodeError:
-            # non-UTF-8 byte streams (synthetic tokens): latin-1 maps every
-            # byte to a DISTINCT char, keeping decode stable and reversible
-            # (utf-8 replacement chars collapse distinct bytes and break
-            # incremental/full decode consistency)
-            return bs.decode("latin-1")
+    @staticmethod
+    def _scan(bs: bytes, final: bool) -> str:
+        """Decode left to right: a complete valid UTF-8 sequence becomes its
+        character; a byte that cannot start or continue one maps to its
+        latin-1 character (every byte to a DISTINCT char, so synthetic
+        token streams stay reversible). A sequence cut off by the end of
+        the input is held back unless `final`. Because a decision about a
+        byte never depends on bytes after its sequence, the output for a
+        prefix is a prefix of the output for the whole stream - which is
+        what streaming needs."""
+        out, i, n = [], 0, len(bs)
+        while i < n:
+            b = bs[i]
+            if b < 0x80:
+                out.append(chr(b))
+                i += 1
+                continue
+            need = (2 if 0xC2 <= b <= 0xDF else 3 if 0xE0 <= b <= 0xEF
+                    else 4 if 0xF0 <= b <= 0xF4 else 0)
+            if need:
+                seq = bs[i:i + need]
+                if len(seq) == need:
+                    try:
+                        out.append(seq.decode("utf-8"))
+                        i += need
+                        continue
+                    except UnicodeDecodeError:
+                        pass
+                elif not final and all(0x80 <= c <= 0xBF for c in seq[1:]):
+                    break       # may still complete: wait for more bytes
+            out.append(chr(b))
+            i += 1
+        return "".join(out)
 
-    def decode_incremental(self, ids: List[int], prev_len: int) -> str:
-        """Decode the new suffix, robust to split UTF-8 sequences."""
-        return self.decode(ids[prev_len:])
+    def decode(self, ids: List[int]) -> str:
+        return self._scan(bytes(i for i in ids if 0 <= i < 256), True)
+
+    def decode_incremental(self, ids: List[int], prev_len: int,
+                           final: bool = False) -> str:
+        """Text that the tokens after `prev_len` add to what was emitted
+        for the first `prev_len`. A trailing incomplete UTF-8 sequence is
+        held back until it completes (or until `final`)."""
+        done = self._scan(bytes(i for i in ids[:prev_len] if 0 <= i < 256),
+                          False)
+        now = self._scan(bytes(i for i in ids if 0 <= i < 256), final)
+        return now[len(done):]
 
 
 class HFTokenizer:

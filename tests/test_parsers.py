@@ -62,7 +62,9 @@ def test_postprocess_combined():
 
 def test_incremental_detok_property():
     """Property: concatenated decode_incremental chunks == full decode,
-    for any token stream and any chunking (streaming-text correctness)."""
+    for any token stream and any chunking (streaming-text correctness).
+    A UTF-8 sequence split by a chunk edge is held back until it completes;
+    the last chunk flushes."""
     from hypothesis import given, settings
     from hypothesis import strategies as st
 
@@ -81,7 +83,8 @@ def test_incremental_detok_property():
             step = cuts[i % len(cuts)]
             i += 1
             nxt = min(len(ids), pos + step)
-            acc += tok.decode_incremental(ids[:nxt], pos)
+            acc += tok.decode_incremental(ids[:nxt], pos,
+                                          final=nxt == len(ids))
             pos = nxt
         assert acc == tok.decode(ids)
 
