@@ -324,8 +324,13 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
   int GS = gsz % 4 == 0 ? 4 : (gsz % 2 == 0 ? 2 : 1);
   if (GS == 4 && T_ * (H / 4) < 256) GS = 2;
   // few rows in flight (decoding): 16 waves split the keys of each row
-  const int NW = T_ * (H / GS) <= 2048 ? 16 : 4;
-  const size_t lds = (size_t)(GS * dk + NW * GS * (2 + dv)) * sizeof(float);
+  int NW = T_ * (H / GS) <= 2048 ? 16 : 4;
+  auto lds_bytes = [&](int gs, int nw) {
+    return (size_t)(gs * dk + nw * gs * (2 + dv)) * sizeof(float);
+  };
+  while (NW > 1 && lds_bytes(GS, NW) > 64 * 1024) NW >>= 1;
+  while (GS > 1 && lds_bytes(GS, NW) > 64 * 1024) GS >>= 1;
+  const size_t lds = lds_bytes(GS, NW);
   TORCH_CHECK(lds <= 64 * 1024,
               "seqmix: attention head sizes exceed the LDS budget");
   const bool vec = (dk * sizeof(T)) % 16 == 0 && dv % 2 == 0 && ps % 16 == 0 &&

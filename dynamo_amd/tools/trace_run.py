@@ -6,8 +6,9 @@ DIR holds config.json and model.safetensors; the model class is chosen from
 config.json as `--model DIR` does everywhere else. Steps arrive on standard
 input, one JSON object a line:
 
-    {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}],
-     "end": []}
+    {"step": 7, "entries": [{"id": "req-1", "tokens": [11, 4], "want": [1]},
+                            {"id": "req-2", "tokens": [9], "want": []}],
+     "end": ["req-2"]}
 
 Each step runs exactly the tokens it brings, all entries as one batch, on
 the cache pages and state slots earlier steps left (LLMEngine.replay_step:
