@@ -41,6 +41,9 @@ struct Geometry {
 inline Geometry geometry(int dk, int dv) {
   Geometry g;
   g.KP = 1;
+  // 16 rows per thread measured slightly faster than 32 for both the
+  // prompt walk and decode; 32 only when the key size needs it
+  while (g.KP * 16 < dk && g.KP < 64) g.KP <<= 1;
   while (g.KP * 32 < dk) g.KP <<= 1;
   TORCH_CHECK(g.KP <= 64, "seqmix: key size too large for the recurrence");
   g.RT = (dk + g.KP - 1) / g.KP <= 16 ? 16 : 32;
@@ -81,16 +84,56 @@ DEVINL float part_sum(float x, int JW) {
   }
 
 // ---------------------------------------------------------------------------
+// Gate pre-passes. The nonlinearities of the gates do not depend on the
+// state, so they run here, parallel over tokens, and the serial walks below
+// only load their results: out[t, h] and out[t, H + h] in fp32.
+//   delta: beta = sigmoid(b); g = exp(-exp(A_log) softplus(a + dt_bias))
+//   mlstm: i = cap tanh((i + ib) / cap); f = logsigmoid(cap tanh((f + fb) / cap))
+template <typename T, bool MLSTM>
+__global__ void gates_kernel(float* __restrict__ out,
+                             const T* __restrict__ proj, int proj_stride,
+                             int off_0, int off_1,
+                             const float* __restrict__ p0,
+                             const float* __restrict__ p1, int H, int total,
+                             float cap) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int t = idx / H, hh = idx - t * H;
+  const float x0 = to_f(proj[(int64_t)t * proj_stride + off_0 + hh]);
+  const float x1 = to_f(proj[(int64_t)t * proj_stride + off_1 + hh]);
+  float y0, y1;
+  if (MLSTM) {
+    y0 = cap * tanhf((x0 + p0[hh]) / cap);
+    y1 = logsigmoid_f(cap * tanhf((x1 + p1[hh]) / cap));
+  } else {
+    y0 = sigmoid_f(x0);
+    y1 = expf(-expf(p0[hh]) * softplus_f(x1 + p1[hh]));
+  }
+  out[(int64_t)t * 2 * H + hh] = y0;
+  out[(int64_t)t * 2 * H + H + hh] = y1;
+}
+
+// RWKV decay w = exp(-exp(wraw + w0)), fp32 [T, H*d]
+template <typename T>
+__global__ void rwkv_decay_kernel(float* __restrict__ out,
+                                  const T* __restrict__ wraw,
+                                  const float* __restrict__ w0, int HD,
+                                  int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  out[idx] = expf(-expf(to_f(wraw[idx]) + w0[idx % HD]));
+}
+
+// ---------------------------------------------------------------------------
 // Gated delta rule. Per token: S <- g S; u = beta (v - S^T k);
 // S <- S + k u^T; o = S^T q. q and k arrive after the short convolution and
 // are made unit vectors here (q also scaled by qscale).
-template <typename T, int PE, int RT>
+template <int PE, int RT>
 __global__ __launch_bounds__(512) void gated_delta_kernel(
     float* __restrict__ out,          // [T, H, dv]
     const float* __restrict__ qkv,    // [T, Cq + Ck + Cv]: unit k, scaled
                                       // unit q, v (after conv + silu)
-    const T* __restrict__ proj, int proj_stride, int off_b, int off_a,
-    const float* __restrict__ A_log, const float* __restrict__ dt_bias,
+    const float* __restrict__ gates,  // [T, 2H]: beta | g
     float* __restrict__ state,        // [slots, H, dk, dv]
     SeqArgs sa, int H, int G, int dk, int dv, int KP) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -112,10 +155,8 @@ __global__ __launch_bounds__(512) void gated_delta_kernel(
   float* sbase = state + ((int64_t)sa.seq_slot[s] * H + hh) * dk * dv;
   float S[RT];
   LOAD_STATE(S, sbase, fresh)
-  const float a_neg = -expf(A_log[hh]);
-  const float dtb = dt_bias[hh];
 
-  struct In { float k[PE], q[PE], braw, araw, vj; };
+  struct In { float k[PE], q[PE], beta, g, vj; };
   In pre[DEPTH];
   const int end = start + len;
   auto fetch = [&](In& in, int t) {
@@ -126,8 +167,8 @@ __global__ __launch_bounds__(512) void gated_delta_kernel(
       in.k[e] = i < dk ? row[Cq + kvh * dk + i] : 0.f;
       in.q[e] = i < dk ? row[kvh * dk + i] : 0.f;
     }
-    in.braw = to_f(proj[(int64_t)t * proj_stride + off_b + hh]);
-    in.araw = to_f(proj[(int64_t)t * proj_stride + off_a + hh]);
+    in.beta = gates[(int64_t)t * 2 * H + hh];
+    in.g = gates[(int64_t)t * 2 * H + H + hh];
     in.vj = valid ? row[2 * Cq + hh * dv + j] : 0.f;
   };
 #pragma unroll
@@ -148,29 +189,30 @@ __global__ __launch_bounds__(512) void gated_delta_kernel(
           ql[i] = pre[u].q[e];
         }
       }
-      const float beta = sigmoid_f(pre[u].braw);
-      const float g = expf(a_neg * softplus_f(pre[u].araw + dtb));
+      const float beta = pre[u].beta;
+      const float g = pre[u].g;
       const float v_cur = pre[u].vj;
       __syncthreads();
       if (t + DEPTH < end) fetch(pre[u], t + DEPTH);
       float kr[RT], qr[RT];
       READ_ROWS(kr, kl)
       READ_ROWS(qr, ql)
-      float dot = 0.f;
+      // four partial sums: the add chain is the token's critical path
+      float d4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < RT; r++) {
         S[r] *= g;
-        dot += S[r] * kr[r];
+        d4[r & 3] += S[r] * kr[r];
       }
-      dot = part_sum(dot, JW);
+      const float dot = part_sum((d4[0] + d4[1]) + (d4[2] + d4[3]), JW);
       const float uu = beta * (v_cur - dot);
-      float o = 0.f;
+      float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < RT; r++) {
         S[r] += kr[r] * uu;
-        o += S[r] * qr[r];
+        o4[r & 3] += S[r] * qr[r];
       }
-      o = part_sum(o, JW);
+      const float o = part_sum((o4[0] + o4[1]) + (o4[2] + o4[3]), JW);
       if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = o;
     }
   }
@@ -199,9 +241,8 @@ __global__ __launch_bounds__(512) void rwkv_kernel(
     float* __restrict__ out,       // [T, H, d]
     const T* __restrict__ r_, const T* __restrict__ k_,
     const T* __restrict__ v_,      // [T, H*d] each
-    const T* __restrict__ wraw,    // [T, H*d]
-    const float* __restrict__ w0,  // [H*d]
-    const float* __restrict__ u,   // [H, d]
+    const float* __restrict__ wdec,  // [T, H*d] decay in (0, 1)
+    const float* __restrict__ u,     // [H, d]
     float* __restrict__ state,     // [slots, H, d, d]
     SeqArgs sa, int H, int dk, int dv, int KP) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -226,12 +267,6 @@ __global__ __launch_bounds__(512) void rwkv_kernel(
     const int rowi = part * RT + r;
     U[r] = rowi < dk ? u[hh * dk + rowi] : 0.f;
   }
-  float w0r[PE];
-#pragma unroll
-  for (int e = 0; e < PE; e++) {
-    const int i = threadIdx.x + e * blockDim.x;
-    w0r[e] = i < dk ? w0[hh * dk + i] : 0.f;
-  }
   const int HD = H * dk;
   struct In { float r[PE], k[PE], w[PE], vj; };
   In pre[DEPTH];
@@ -243,7 +278,7 @@ __global__ __launch_bounds__(512) void rwkv_kernel(
       const int i = threadIdx.x + e * blockDim.x;
       in.r[e] = i < dk ? to_f(r_[base + i]) : 0.f;
       in.k[e] = i < dk ? to_f(k_[base + i]) : 0.f;
-      in.w[e] = i < dk ? to_f(wraw[base + i]) : 0.f;
+      in.w[e] = i < dk ? wdec[base + i] : 0.f;
     }
     in.vj = valid ? to_f(v_[(int64_t)t * H * dv + hh * dv + j]) : 0.f;
   };
@@ -264,7 +299,7 @@ __global__ __launch_bounds__(512) void rwkv_kernel(
         if (i < DKP) {
           rl[i] = pre[u].r[e];
           kl[i] = pre[u].k[e];
-          wl[i] = expf(-expf(pre[u].w[e] + w0r[e]));
+          wl[i] = pre[u].w[e];
         }
       }
       const float v_cur = pre[u].vj;
@@ -274,14 +309,14 @@ __global__ __launch_bounds__(512) void rwkv_kernel(
       READ_ROWS(rr, rl)
       READ_ROWS(kr, kl)
       READ_ROWS(wr, wl)
-      float o = 0.f;
+      float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < RT; r++) {
         const float kv = kr[r] * v_cur;
-        o += rr[r] * (S[r] + U[r] * kv);
+        o4[r & 3] += rr[r] * (S[r] + U[r] * kv);
         S[r] = wr[r] * S[r] + kv;
       }
-      o = part_sum(o, JW);
+      const float o = part_sum((o4[0] + o4[1]) + (o4[2] + o4[3]), JW);
       if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = o;
     }
   }
@@ -297,13 +332,11 @@ template <typename T, int PE, int RT>
 __global__ __launch_bounds__(512) void mlstm_kernel(
     float* __restrict__ out,  // [T, H, dv]
     const T* __restrict__ proj, int proj_stride, int off_q, int off_k,
-    int off_v, int off_i, int off_f, const float* __restrict__ i_bias,
-    const float* __restrict__ f_bias,
+    int off_v, const float* __restrict__ gates,  // [T, 2H]: i | f (log)
     float* __restrict__ state_S,        // [slots, H, dk, dv]
     const float* __restrict__ state_n,  // [slots, H, dk]
     const float* __restrict__ state_m,  // [slots, H]
-    SeqArgs sa, int H, int dk, int dv, int KP, float qscale, float cap,
-    float den_eps) {
+    SeqArgs sa, int H, int dk, int dv, int KP, float qscale, float den_eps) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // [2 buffers][k | q][DKP]
   const int DKP = KP * RT;
@@ -329,9 +362,8 @@ __global__ __launch_bounds__(512) void mlstm_kernel(
     N[r] = (!fresh && rowi < dk) ? nbase[rowi] : 0.f;
   }
   float m = fresh ? 0.f : state_m[slot * H + hh];
-  const float ib = i_bias[hh], fb = f_bias[hh];
 
-  struct In { float k[PE], q[PE], iraw, fraw, vj; };
+  struct In { float k[PE], q[PE], ig, fg, vj; };
   In pre[DEPTH];
   const int end = start + len;
   auto fetch = [&](In& in, int t) {
@@ -342,8 +374,8 @@ __global__ __launch_bounds__(512) void mlstm_kernel(
       in.k[e] = i < dk ? to_f(row[off_k + hh * dk + i]) : 0.f;
       in.q[e] = i < dk ? to_f(row[off_q + hh * dk + i]) * qscale : 0.f;
     }
-    in.iraw = to_f(row[off_i + hh]);
-    in.fraw = to_f(row[off_f + hh]);
+    in.ig = gates[(int64_t)t * 2 * H + hh];
+    in.fg = gates[(int64_t)t * 2 * H + H + hh];
     in.vj = valid ? to_f(row[off_v + hh * dv + j]) : 0.f;
   };
 #pragma unroll
@@ -364,8 +396,8 @@ __global__ __launch_bounds__(512) void mlstm_kernel(
           ql[i] = pre[u].q[e];
         }
       }
-      const float ig = cap * tanhf((pre[u].iraw + ib) / cap);
-      const float fg = logsigmoid_f(cap * tanhf((pre[u].fraw + fb) / cap));
+      const float ig = pre[u].ig;
+      const float fg = pre[u].fg;
       const float v_cur = pre[u].vj;
       __syncthreads();
       if (t + DEPTH < end) fetch(pre[u], t + DEPTH);
@@ -375,17 +407,17 @@ __global__ __launch_bounds__(512) void mlstm_kernel(
       float kr[RT], qr[RT];
       READ_ROWS(kr, kl)
       READ_ROWS(qr, ql)
-      float num = 0.f, nq = 0.f;
+      float n4[4] = {0.f, 0.f, 0.f, 0.f}, q4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < RT; r++) {
         const float bk = b * kr[r];
         S[r] = a * S[r] + bk * v_cur;
         N[r] = a * N[r] + bk;
-        num += S[r] * qr[r];
-        nq += N[r] * qr[r];
+        n4[r & 3] += S[r] * qr[r];
+        q4[r & 3] += N[r] * qr[r];
       }
-      num = part_sum(num, JW);
-      nq = part_sum(nq, JW);
+      const float num = part_sum((n4[0] + n4[1]) + (n4[2] + n4[3]), JW);
+      const float nq = part_sum((q4[0] + q4[1]) + (q4[2] + q4[3]), JW);
       const float den = fmaxf(fabsf(nq), expf(-m)) + den_eps;
       if (valid && part == 0) out[((int64_t)t * H + hh) * dv + j] = num / den;
     }
@@ -398,10 +430,9 @@ __global__ __launch_bounds__(512) void mlstm_kernel(
 // the same gates once per (sequence, head) and stores the new n and m.
 template <typename T>
 __global__ void mlstm_nm_kernel(
-    const T* __restrict__ proj, int proj_stride, int off_k, int off_i,
-    int off_f, const float* __restrict__ i_bias,
-    const float* __restrict__ f_bias, float* __restrict__ state_n,
-    float* __restrict__ state_m, SeqArgs sa, int H, int dk, float cap) {
+    const T* __restrict__ proj, int proj_stride, int off_k,
+    const float* __restrict__ gates, float* __restrict__ state_n,
+    float* __restrict__ state_m, SeqArgs sa, int H, int dk) {
   const int s = blockIdx.x, hh = blockIdx.y;
   const int len = sa.seq_len[s];
   if (len == 0) return;
@@ -410,16 +441,14 @@ __global__ void mlstm_nm_kernel(
   const int slot = sa.seq_slot[s];
   float* nbase = state_n + ((int64_t)slot * H + hh) * dk;
   float m0 = fresh ? 0.f : state_m[slot * H + hh];
-  const float ib = i_bias[hh], fb = f_bias[hh];
   float m_end = m0;  // same on every thread; thread 0 owns row 0
   for (int i = threadIdx.x; i < dk; i += blockDim.x) {
     float n = fresh ? 0.f : nbase[i];
     float m = m0;
     for (int t = start; t < start + len; t++) {
       const T* row = proj + (int64_t)t * proj_stride;
-      const float ig = cap * tanhf((to_f(row[off_i + hh]) + ib) / cap);
-      const float fg =
-          logsigmoid_f(cap * tanhf((to_f(row[off_f + hh]) + fb) / cap));
+      const float ig = gates[(int64_t)t * 2 * H + hh];
+      const float fg = gates[(int64_t)t * 2 * H + H + hh];
       const float mn = fmaxf(fg + m, ig);
       n = expf(fg + m - mn) * n + expf(ig - mn) * to_f(row[off_k + hh * dk + i]);
       m = mn;
@@ -437,6 +466,11 @@ __global__ void mlstm_nm_kernel(
   ((g).DKP <= (g).NW * 64                                                    \
        ? ((g).RT == 16 ? K<T, 1, 16> : K<T, 1, 32>)                          \
        : ((g).RT == 16 ? K<T, PEMAX, 16> : K<T, PEMAX, 32>))
+
+#define PICK_KERNEL_F32(K, g)                                                \
+  ((g).DKP <= (g).NW * 64                                                    \
+       ? ((g).RT == 16 ? K<1, 16> : K<1, 32>)                                \
+       : ((g).RT == 16 ? K<PEMAX, 16> : K<PEMAX, 32>))
 
 SeqArgs seq_args(const torch::Tensor& seq_start, const torch::Tensor& seq_len,
                  const torch::Tensor& seq_slot, const torch::Tensor& seq_pos0,
@@ -482,12 +516,17 @@ void gated_delta_rule(torch::Tensor out, torch::Tensor qkv, torch::Tensor proj,
   hipLaunchKernelGGL(unit_heads_kernel, dim3(T_, 2 * (int)G), dim3(64), 0,
                      cur_stream(), ptr<float>(qkv), (int)qkv.size(1), (int)G,
                      dk, (float)qscale, (float)unit_eps);
+  torch::Tensor gates = torch::empty({T_, 2 * H}, out.options());
   DISPATCH_ACT(proj, hipLaunchKernelGGL(
-      PICK_KERNEL(gated_delta_kernel, g), dim3(B, H, g.tiles),
-      dim3(g.NW * 64), 4 * g.DKP * sizeof(float), cur_stream(),
-      ptr<float>(out), cptr<float>(qkv), cptr<T>(proj), (int)proj.stride(0),
-      (int)off_b, (int)off_a, cptr<float>(A_log), cptr<float>(dt_bias),
-      ptr<float>(state), sa, H, (int)G, dk, dv, g.KP););
+      (gates_kernel<T, false>), dim3((T_ * H + 255) / 256), dim3(256), 0,
+      cur_stream(), ptr<float>(gates), cptr<T>(proj), (int)proj.stride(0),
+      (int)off_b, (int)off_a, cptr<float>(A_log), cptr<float>(dt_bias), H,
+      T_ * H, 0.f););
+  hipLaunchKernelGGL(PICK_KERNEL_F32(gated_delta_kernel, g),
+                     dim3(B, H, g.tiles), dim3(g.NW * 64),
+                     4 * g.DKP * sizeof(float), cur_stream(), ptr<float>(out),
+                     cptr<float>(qkv), cptr<float>(gates), ptr<float>(state),
+                     sa, H, (int)G, dk, dv, g.KP);
 }
 
 void rwkv_time_mix(torch::Tensor out, torch::Tensor r, torch::Tensor k,
@@ -512,11 +551,18 @@ void rwkv_time_mix(torch::Tensor out, torch::Tensor r, torch::Tensor k,
   if (T_ == 0 || B == 0) return;
   SeqArgs sa = seq_args(seq_start, seq_len, seq_slot, seq_pos0, state.size(0));
   Geometry g = geometry(dk, dv);
-  DISPATCH_ACT(r, hipLaunchKernelGGL(
-      PICK_KERNEL(rwkv_kernel, g), dim3(B, H, g.tiles), dim3(g.NW * 64),
-      6 * g.DKP * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(r),
-      cptr<T>(k), cptr<T>(v), cptr<T>(wraw), cptr<float>(w0), cptr<float>(u),
-      ptr<float>(state), sa, H, dk, dv, g.KP););
+  torch::Tensor wdec = torch::empty({T_, H * dk}, out.options());
+  const int64_t nw = (int64_t)T_ * H * dk;
+  DISPATCH_ACT(r, {
+    hipLaunchKernelGGL(rwkv_decay_kernel<T>, dim3((nw + 255) / 256), dim3(256),
+                       0, cur_stream(), ptr<float>(wdec), cptr<T>(wraw),
+                       cptr<float>(w0), H * dk, nw);
+    hipLaunchKernelGGL(
+        PICK_KERNEL(rwkv_kernel, g), dim3(B, H, g.tiles), dim3(g.NW * 64),
+        6 * g.DKP * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(r),
+        cptr<T>(k), cptr<T>(v), cptr<float>(wdec), cptr<float>(u),
+        ptr<float>(state), sa, H, dk, dv, g.KP);
+  });
 }
 
 void mlstm_memory(torch::Tensor out, torch::Tensor proj, int64_t off_q,
@@ -549,16 +595,25 @@ void mlstm_memory(torch::Tensor out, torch::Tensor proj, int64_t off_q,
   if (T_ == 0 || B == 0) return;
   SeqArgs sa = seq_args(seq_start, seq_len, seq_slot, seq_pos0, state_S.size(0));
   Geometry g = geometry(dk, dv);
-  DISPATCH_ACT(proj, hipLaunchKernelGGL(
-      PICK_KERNEL(mlstm_kernel, g), dim3(B, H, g.tiles), dim3(g.NW * 64),
-      4 * g.DKP * sizeof(float), cur_stream(), ptr<float>(out), cptr<T>(proj),
-      (int)proj.stride(0), (int)off_q, (int)off_k, (int)off_v, (int)off_i,
-      (int)off_f, cptr<float>(i_bias), cptr<float>(f_bias),
-      ptr<float>(state_S), ptr<float>(state_n), ptr<float>(state_m), sa, H, dk,
-      dv, g.KP, (float)qscale, (float)cap, (float)den_eps);
+  torch::Tensor gates = torch::empty({T_, 2 * H}, out.options());
+  DISPATCH_ACT(proj, {
+    hipLaunchKernelGGL((gates_kernel<T, true>), dim3((T_ * H + 255) / 256),
+                       dim3(256), 0, cur_stream(), ptr<float>(gates),
+                       cptr<T>(proj), (int)proj.stride(0), (int)off_i,
+                       (int)off_f, cptr<float>(i_bias), cptr<float>(f_bias), H,
+                       T_ * H, (float)cap);
     hipLaunchKernelGGL(
-      mlstm_nm_kernel<T>, dim3(B, H), dim3(dk < 64 ? 64 : (dk > 256 ? 256 : (dk + 63) / 64 * 64)),
-      0, cur_stream(), cptr<T>(proj), (int)proj.stride(0), (int)off_k,
-      (int)off_i, (int)off_f, cptr<float>(i_bias), cptr<float>(f_bias),
-      ptr<float>(state_n), ptr<float>(state_m), sa, H, dk, (float)cap););
+        PICK_KERNEL(mlstm_kernel, g), dim3(B, H, g.tiles), dim3(g.NW * 64),
+        4 * g.DKP * sizeof(float), cur_stream(), ptr<float>(out),
+        cptr<T>(proj), (int)proj.stride(0), (int)off_q, (int)off_k,
+        (int)off_v, cptr<float>(gates), ptr<float>(state_S),
+        ptr<float>(state_n), ptr<float>(state_m), sa, H, dk, dv, g.KP,
+        (float)qscale, (float)den_eps);
+    hipLaunchKernelGGL(
+        mlstm_nm_kernel<T>, dim3(B, H),
+        dim3(dk < 64 ? 64 : (dk > 256 ? 256 : (dk + 63) / 64 * 64)), 0,
+        cur_stream(), cptr<T>(proj), (int)proj.stride(0), (int)off_k,
+        cptr<float>(gates), ptr<float>(state_n), ptr<float>(state_m), sa, H,
+        dk);
+  });
 }
