@@ -44,6 +44,13 @@ void biased_attention(Tensor out, Tensor proj, int64_t off_q, Tensor kcache,
                       Tensor positions, Tensor seq_len, OptTensor r1,
                       OptTensor r2, double scale, double temp_coef,
                       int64_t temp_every);
+bool biased_attention_mfma_supported(int64_t dk, int64_t dv);
+void biased_attention_mfma(Tensor out, Tensor proj, int64_t off_q,
+                           Tensor kcache, Tensor vcache, Tensor page_table,
+                           Tensor tile_row0, Tensor tile_rows,
+                           int64_t max_tile_rows, Tensor tok_seq,
+                           Tensor positions, OptTensor r1, OptTensor r2,
+                           double scale, double temp_coef, int64_t temp_every);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "dynamo_amd sequence-mixer kernels (gfx950)";
@@ -60,4 +67,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("mlstm_memory", &mlstm_memory);
   m.def("kv_append_norm", &kv_append_norm);
   m.def("biased_attention", &biased_attention);
+  m.def("biased_attention_mfma_supported", &biased_attention_mfma_supported);
+  m.def("biased_attention_mfma", &biased_attention_mfma);
 }

@@ -215,8 +215,14 @@ class ModelRunner:
         from dynamo_amd.ops.seq import SeqBatch
         dev = self.device
         spans, tok_seq = [], []
+        tile_row0, tile_rows = [], []
+        nd = len(sched.decodes)
         row = 0
-        for ss in sched.decodes + sched.prefills:
+        for k, ss in enumerate(sched.decodes + sched.prefills):
+            if k >= nd:     # prompt portion: tiles of 64 rows
+                for q0 in range(0, ss.n_new, 64):
+                    tile_row0.append(row + q0)
+                    tile_rows.append(min(64, ss.n_new - q0))
             r = ss.req
             if r.state_slot is None:
                 raise RuntimeError(f"{r.req_id} runs without a state slot")
@@ -234,7 +240,11 @@ class ModelRunner:
                 dev, non_blocking=True),
             seq_start=cols[0], seq_len=cols[1], seq_slot=cols[2],
             seq_pos0=cols[3], page_table=pt.to(dev, non_blocking=True),
-            host=spans)
+            host=spans, num_decode=nd,
+            tiles=(torch.tensor(tile_row0, dtype=torch.int32).to(
+                       dev, non_blocking=True),
+                   torch.tensor(tile_rows, dtype=torch.int32).to(
+                       dev, non_blocking=True)))
 
     # ------------------------------------------------------------------
     @torch.inference_mode()

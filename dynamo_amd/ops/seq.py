@@ -45,6 +45,12 @@ class SeqBatch:
     seq_slot: torch.Tensor     # [B] int32: recurrent-state slot
     seq_pos0: torch.Tensor     # [B] int32: position of the first row
     page_table: Optional[torch.Tensor] = None   # [B, maxp] int32
+    # rows [0, num_decode) are single decoded tokens; the prompt portions
+    # after them are also listed as tiles of at most 64 rows of one
+    # sequence: (first row [NT], rows [NT]) int32, for the matrix-core
+    # attention kernel. None = no tiling (every row takes the row kernel).
+    num_decode: int = 0
+    tiles: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
     # host copy [(start, len, slot, pos0)] for the CPU path
     host: Optional[List[Tuple[int, int, int, int]]] = None
 
@@ -202,12 +208,28 @@ def biased_attention(proj, off_q: int, H: int, kcache, vcache, positions,
     """-> [T, H*dv] in proj's dtype."""
     dv = vcache.shape[3]
     if proj.is_cuda:
-        out = torch.empty(proj.shape[0], H, dv, dtype=proj.dtype,
-                          device=proj.device)
-        hip_seq().biased_attention(out, proj, off_q, kcache, vcache,
-                                   sb.page_table, sb.tok_seq, positions,
-                                   sb.seq_len, r1, r2, float(scale),
-                                   float(temp_coef), int(temp_every))
-        return out.view(proj.shape[0], H * dv)
+        T = proj.shape[0]
+        out = torch.empty(T, H, dv, dtype=proj.dtype, device=proj.device)
+        m = hip_seq()
+        # prompt portions in bf16 go to the MFMA kernel when the head sizes
+        # fit it; decoded tokens, fp32 and other sizes take the row kernel
+        tiled = (sb.tiles is not None and proj.dtype == torch.bfloat16
+                 and m.biased_attention_mfma_supported(kcache.shape[3], dv)
+                 and kcache.data_ptr() % 16 == 0
+                 and vcache.data_ptr() % 16 == 0)
+        nrow = sb.num_decode if tiled else T
+        if nrow:
+            m.biased_attention(out[:nrow], proj[:nrow], off_q, kcache, vcache,
+                               sb.page_table, sb.tok_seq[:nrow],
+                               positions[:nrow], sb.seq_len, r1, r2,
+                               float(scale), float(temp_coef),
+                               int(temp_every))
+        if tiled and sb.tiles[0].numel():
+            m.biased_attention_mfma(out, proj, off_q, kcache, vcache,
+                                    sb.page_table, sb.tiles[0], sb.tiles[1],
+                                    64, sb.tok_seq, positions, r1, r2,
+                                    float(scale), float(temp_coef),
+                                    int(temp_every))
+        return out.view(T, H * dv)
     return seq_ref.biased_attention(proj, off_q, H, kcache, vcache, positions,
                                     sb, r1, r2, scale, temp_coef, temp_every)

@@ -142,7 +142,10 @@ def test_recurrences(dk, dv):
 
 @pytest.mark.parametrize("H,G,dk,dv,ps", [(6, 3, 24, 40, 16), (3, 1, 10, 7, 8),
                                           (8, 2, 128, 128, 64),
-                                          (4, 4, 64, 300, 16)])
+                                          (4, 4, 64, 300, 16),
+                                          (4, 2, 96, 96, 16),
+                                          (2, 1, 200, 64, 64),
+                                          (2, 2, 40, 256, 8)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention(H, G, dk, dv, ps, dtype):
     g = torch.Generator().manual_seed(3)
@@ -176,3 +179,24 @@ def test_attention(H, G, dk, dv, ps, dtype):
     for a, b in zip(*outs):
         assert torch.allclose(a, b, atol=tol, rtol=1e-3), \
             float((a - b).abs().max())
+    if dtype == torch.bfloat16 and sops.hip_seq().biased_attention_mfma_supported(dk, dv):
+        # the matrix-core kernel on the same cache: the 70-row and 9-row
+        # portions as tiles (64 + 6, 9), the single row on the row kernel
+        # in between; against the row kernel it differs only by the bf16
+        # rounding of the softmax weights
+        order = [1, 0, 2]                      # decoded row first
+        spans2 = [spans[i] for i in order]
+        sb, _ = _batch(spans2, DEV)
+        sb.page_table = perm[order].to(torch.int32).to(DEV)
+        rows = torch.cat([torch.arange(70, 71), torch.arange(0, 70),
+                          torch.arange(71, 80)])
+        sb.num_decode = 1
+        sb.tiles = (torch.tensor([1, 65, 71], dtype=torch.int32, device=DEV),
+                    torch.tensor([64, 6, 9], dtype=torch.int32, device=DEV))
+        o2 = sops.biased_attention(
+            proj[rows].to(DEV), 0, H, k_, v_,
+            torch.tensor(pos, dtype=torch.int32)[rows].to(DEV), sb,
+            r1.to(DEV), r2.to(DEV), 0.2, 0.7, 16).float().cpu()
+        ref = outs[1][0][rows]
+        assert torch.allclose(o2, ref, atol=2e-2, rtol=2e-2), \
+            float((o2 - ref).abs().max())
