@@ -114,8 +114,10 @@ __global__ __launch_bounds__(256) void biased_attention_mfma_kernel(
       }
       *reinterpret_cast<short8_t*>(k_lds + row * KS + v * 8) = x;
     }
+    // consecutive threads take consecutive keys of one channel group, so
+    // the transposed 2-byte LDS writes fall in consecutive banks
     for (int slot = threadIdx.x; slot < BN * vvecs; slot += 256) {
-      const int row = slot / vvecs, v = slot - row * vvecs;
+      const int v = slot / BN, row = slot - v * BN;
       const int j = t0 + row;
       short8_t x{};
       if (j < kv_end && v * 8 < dv) {
