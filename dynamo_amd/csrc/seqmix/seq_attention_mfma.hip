@@ -9,7 +9,8 @@
 // transposed (channel-major) so that the B operand of the second product
 // is a 16-byte run of keys. The fp32 scores get the row's temperature and
 // scale, the log distance penalty and the causal mask, then an online
-// softmax; the weights pass through LDS (bf16) to become the A operand.
+// softmax; the weights pass through LDS as a bf16 hi + lo pair to become
+// the A operand of two products.
 //
 // Fragment layouts of mfma_f32_16x16x32_bf16 (lane l, lr = l % 16,
 // lg = l / 16):  A: A[row = lr][k = 8 lg + i], i = 0..7
@@ -180,25 +181,39 @@ __global__ __launch_bounds__(256) void biased_attention_mfma_kernel(
 #pragma unroll
       for (int d = 0; d < DN; d++) acc_o[d][r] *= corr;
     }
-    // ---- weights to LDS in the A layout of the second product
+    // ---- weights to LDS in the A layout of the second product, as a
+    // bf16 pair hi + lo (about 16 bits of mantissa, so the product below
+    // sees the fp32 weights almost exactly). lo reuses the K block, which
+    // every wave has finished reading once the barrier is passed.
+    __syncthreads();
     short* pw = p_lds + wid * 16 * VS;
+    short* pl = k_lds + wid * 16 * VS;
 #pragma unroll
     for (int r = 0; r < 4; r++)
 #pragma unroll
-      for (int n = 0; n < 4; n++)
-        pw[(lg * 4 + r) * VS + n * 16 + lr] = (short)from_f<bf16_t>(p[n][r]);
+      for (int n = 0; n < 4; n++) {
+        const bf16_t hi = from_f<bf16_t>(p[n][r]);
+        const bf16_t lo = from_f<bf16_t>(p[n][r] - to_f(hi));
+        pw[(lg * 4 + r) * VS + n * 16 + lr] = (short)hi;
+        pl[(lg * 4 + r) * VS + n * 16 + lr] = (short)lo;
+      }
     __syncthreads();
     // ---- O += P V
 #pragma unroll
     for (int kt = 0; kt < 2; kt++) {
       short8_t pa = *reinterpret_cast<const short8_t*>(
           pw + lr * VS + kt * 32 + lg * 8);
+      short8_t pb = *reinterpret_cast<const short8_t*>(
+          pl + lr * VS + kt * 32 + lg * 8);
 #pragma unroll
       for (int d = 0; d < DN; d++) {
         short8_t vb = *reinterpret_cast<const short8_t*>(
             vt_lds + (d * 16 + lr) * VS + kt * 32 + lg * 8);
         acc_o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
             *reinterpret_cast<bf16x8_t*>(&pa),
+            *reinterpret_cast<bf16x8_t*>(&vb), acc_o[d], 0, 0, 0);
+        acc_o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            *reinterpret_cast<bf16x8_t*>(&pb),
             *reinterpret_cast<bf16x8_t*>(&vb), acc_o[d], 0, 0, 0);
       }
     }
