@@ -10,6 +10,16 @@
 //
 // The same kernel serves prompt portions and decoded tokens: a row only
 // needs its position and its sequence's page table.
+//
+// The kernel is general in three more ways, which paged_attention_rows
+// exposes: a sliding window (row i sees keys j with 0 <= i - j < window),
+// several key maps per kv head (the cached key row of a kv head holds
+// `kmaps` keys of size dk back to back; query head h has one query per map,
+// laid out [h][map][dk], and every map is a softmax attention of its own
+// over the same values - the output is [T, H, kmaps, dv]), and a value row
+// stride of its own, so values may alias a prefix of the key rows (latent
+// attention, where the cached latent is both key part and value). The
+// output may be fp32 whatever the cache type.
 #include "seq_common.h"
 
 namespace {
@@ -79,16 +89,17 @@ template <> struct Vec16<bf16_t> {
 // clamped into range instead of tested, so the loads of a pass issue back
 // to back. Otherwise a plain scalar path runs. EVT is the number of value
 // channels a lane owns.
-template <typename T, int GS, bool FAST, int EVT>
+template <typename T, typename TO, int GS, bool FAST, int EVT>
 __global__ __launch_bounds__(1024) void biased_attention_kernel(
-    T* __restrict__ out,  // [T, H, dv]
+    TO* __restrict__ out,  // [T, H, kmaps, dv]
     const T* __restrict__ proj, int proj_stride, int off_q,
     const T* __restrict__ kcache, const T* __restrict__ vcache,
     const int* __restrict__ page_table, int table_stride,
     const int* __restrict__ tok_seq, const int* __restrict__ positions,
     const int* __restrict__ seq_len, const float* __restrict__ r1,
     const float* __restrict__ r2, int H, int G, int dk, int dv, int ps,
-    float scale, float temp_coef, int temp_every, int has_bias) {
+    float scale, float temp_coef, int temp_every, int has_bias, int kmaps,
+    int vrow, int window) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // q [GS][dk]; merge [waves][GS][2 + dv]
   constexpr int VN = Vec16<T>::N;
@@ -96,8 +107,12 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
   const int nwv = blockDim.x >> 6;
   const int s = tok_seq[t];
   if (seq_len[s] == 0) return;  // padding row
-  const int h0 = blockIdx.y * GS;  // first query head of this group
-  const int g = h0 / (H / G);
+  // blockIdx.y = ((kv head * kmaps) + map) * (blocks per kv head) + block
+  const int gsz = H / G, bpg = gsz / GS;
+  const int g = blockIdx.y / (kmaps * bpg);
+  const int map = (blockIdx.y / bpg) % kmaps;
+  const int h0 = g * gsz + (blockIdx.y % bpg) * GS;  // first query head
+  const int krow = kmaps * dk, koff = map * dk;
   const int pos = positions[t];
   float temp = 1.f;
   if (temp_coef != 0.f)
@@ -105,8 +120,11 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
   const float qmul = temp * scale;
   float* qs = lds;
   float* mg = lds + GS * dk;
-  for (int i = threadIdx.x; i < GS * dk; i += blockDim.x)
-    qs[i] = to_f(proj[(int64_t)t * proj_stride + off_q + h0 * dk + i]) * qmul;
+  for (int i = threadIdx.x; i < GS * dk; i += blockDim.x) {
+    const int a = i / dk, e = i - a * dk;
+    qs[i] = to_f(proj[(int64_t)t * proj_stride + off_q +
+                      ((h0 + a) * kmaps + map) * dk + e]) * qmul;
+  }
   __syncthreads();
   const int* table = page_table + (int64_t)s * table_stride;
   float b1[GS], b2[GS];
@@ -129,8 +147,9 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
     for (int e = 0; e < EVT; e++) acc[a][e] = 0.f;
   }
   const int ctx = pos + 1;
+  const int jmin = window > 0 ? max(0, ctx - window) : 0;  // first visible key
   const int nchunks = (ctx + 63) >> 6;
-  for (int c = wave; c < nchunks; c += nwv) {
+  for (int c = (jmin >> 6) + wave; c < nchunks; c += nwv) {
     const int j0 = c << 6;
     // ---- scores: pass p covers keys j0 + 16 p + quad ----
     float sc[4][GS];
@@ -142,7 +161,7 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
 #pragma unroll
       for (int a = 0; a < GS; a++) d[a] = 0.f;
       const int64_t page = table[jc / ps];
-      const T* k = kcache + ((page * G + g) * ps + (jc % ps)) * dk;
+      const T* k = kcache + ((page * G + g) * ps + (jc % ps)) * krow + koff;
       if (FAST) {
         for (int v0 = qq; v0 < nvec; v0 += 16) {
           Vec16<T> kv[4];
@@ -182,7 +201,7 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
         x += __shfl_xor(x, 1, 64);
         x += __shfl_xor(x, 2, 64);
         if (has_bias) x -= b1[a] * log1pf(b2[a] * (float)(pos - jc));
-        sc[p][a] = j < ctx ? x : -INFINITY;
+        sc[p][a] = (j < ctx && j >= jmin) ? x : -INFINITY;
       }
     }
     // ---- online softmax (every lane of a quad holds the same score) ----
@@ -214,14 +233,15 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
         // the 16 keys of a pass lie in one page; rows past the context
         // are read from the last valid row and weigh 0
         const T* vrun =
-            vcache + (((int64_t)table[jp / ps] * G + g) * ps + (jp % ps)) * dv;
+            vcache +
+            (((int64_t)table[jp / ps] * G + g) * ps + (jp % ps)) * vrow;
 #pragma unroll
         for (int k0 = 0; k0 < 16; k0 += 8) {
           if (k0 >= nk) break;
           float vf[8][EVT];
 #pragma unroll
           for (int u = 0; u < 8; u++) {
-            const T* v = vrun + (int64_t)min(k0 + u, nk - 1) * dv;
+            const T* v = vrun + (int64_t)min(k0 + u, nk - 1) * vrow;
 #pragma unroll
             for (int e = 0; e < EVT; e += 2) {
               const int ch = min((e / 2) * 128 + 2 * lane, dv - 2);
@@ -252,8 +272,8 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
       } else {
         for (int kk = 0; kk < nk; kk++) {
           const int j = jp + kk;
-          const T* v =
-              vcache + (((int64_t)table[j / ps] * G + g) * ps + (j % ps)) * dv;
+          const T* v = vcache +
+              (((int64_t)table[j / ps] * G + g) * ps + (j % ps)) * vrow;
           float w[GS];
 #pragma unroll
           for (int a = 0; a < GS; a++) w[a] = __shfl(pr[p][a], kk << 2, 64);
@@ -303,28 +323,34 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
         const float mw = mg[(w * GS + a) * MS];
         if (mw != -INFINITY) o += expf(mw - mx) * mg[(w * GS + a) * MS + 2 + ch];
       }
-      out[((int64_t)t * H + h0 + a) * dv + ch] = from_f<T>(o * inv);
+      out[(((int64_t)t * H + h0 + a) * kmaps + map) * dv + ch] =
+          from_f<TO>(o * inv);
     }
   }
 }
 
-template <typename T>
+template <typename T, typename TO>
 void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
-                      torch::Tensor& kcache, torch::Tensor& vcache,
+                      torch::Tensor& kcache, const void* vptr, int dv, int vrow,
                       torch::Tensor& page_table, torch::Tensor& tok_seq,
                       torch::Tensor& positions, torch::Tensor& seq_len,
                       c10::optional<torch::Tensor>& r1,
                       c10::optional<torch::Tensor>& r2, double scale,
-                      double temp_coef, int64_t temp_every) {
-  const int T_ = out.size(0), H = out.size(1), dv = out.size(2);
-  const int G = kcache.size(1), ps = kcache.size(2), dk = kcache.size(3);
+                      double temp_coef, int64_t temp_every, int kmaps,
+                      int window) {
+  const int T_ = out.size(0), H = out.size(1);
+  const int G = kcache.size(1), ps = kcache.size(2);
+  const int dk = kcache.size(3) / kmaps;
   const int gsz = H / G;
   // heads of a group share each key/value load; with few rows in flight a
   // smaller group gives the chip more workgroups instead
   int GS = gsz % 4 == 0 ? 4 : (gsz % 2 == 0 ? 2 : 1);
-  if (GS == 4 && T_ * (H / 4) < 256) GS = 2;
-  // few rows in flight (decoding): 16 waves split the keys of each row
-  int NW = T_ * (H / GS) <= 2048 ? 16 : 4;
+  if (GS == 4 && T_ * (H * kmaps / 4) < 256) GS = 2;
+  // few rows in flight (decoding): 16 waves split the keys of each row; a
+  // window bounds the keys of a row, and the waves with them
+  int NW = T_ * (H * kmaps / GS) <= 2048 ? 16 : 4;
+  if (window > 0)
+    while (NW > 1 && (NW - 1) * 64 >= window + 63) NW >>= 1;
   auto lds_bytes = [&](int gs, int nw) {
     return (size_t)(gs * dk + nw * gs * (2 + dv)) * sizeof(float);
   };
@@ -334,18 +360,20 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
   TORCH_CHECK(lds <= 64 * 1024,
               "seqmix: attention head sizes exceed the LDS budget");
   const bool vec = (dk * sizeof(T)) % 16 == 0 && dv % 2 == 0 && ps % 16 == 0 &&
+                   vrow % 2 == 0 &&
                    reinterpret_cast<uintptr_t>(kcache.data_ptr()) % 16 == 0 &&
-                   reinterpret_cast<uintptr_t>(vcache.data_ptr()) % 8 == 0;
+                   reinterpret_cast<uintptr_t>(vptr) % 8 == 0;
   const bool small = dv <= 128;
 #define LAUNCH_ATT(GS_, VEC_, EVT_)                                         \
-  hipLaunchKernelGGL((biased_attention_kernel<T, GS_, VEC_, EVT_>),         \
-      dim3(T_, H / GS_), dim3(NW * 64), lds, cur_stream(), ptr<T>(out),     \
-      cptr<T>(proj), (int)proj.stride(0), (int)off_q, cptr<T>(kcache),      \
-      cptr<T>(vcache), cptr<int>(page_table), (int)page_table.stride(0),    \
+  hipLaunchKernelGGL((biased_attention_kernel<T, TO, GS_, VEC_, EVT_>),     \
+      dim3(T_, H * kmaps / GS_), dim3(NW * 64), lds, cur_stream(),          \
+      ptr<TO>(out), cptr<T>(proj), (int)proj.stride(0), (int)off_q,         \
+      cptr<T>(kcache), reinterpret_cast<const T*>(vptr),                    \
+      cptr<int>(page_table), (int)page_table.stride(0),                     \
       cptr<int>(tok_seq), cptr<int>(positions), cptr<int>(seq_len),         \
       r1 ? cptr<float>(*r1) : nullptr, r2 ? cptr<float>(*r2) : nullptr, H,  \
       G, dk, dv, ps, (float)scale, (float)temp_coef, (int)temp_every,       \
-      r1 ? 1 : 0)
+      r1 ? 1 : 0, kmaps, vrow, window)
 #define LAUNCH_GS(GS_)                                                      \
   do {                                                                      \
     if (vec && small) LAUNCH_ATT(GS_, true, 2);                             \
@@ -387,24 +415,49 @@ void kv_append_norm(torch::Tensor kcache, torch::Tensor vcache,
       vnorm ? 1 : 0, (float)eps););
 }
 
-void biased_attention(torch::Tensor out, torch::Tensor proj, int64_t off_q,
-                      torch::Tensor kcache, torch::Tensor vcache,
-                      torch::Tensor page_table, torch::Tensor tok_seq,
-                      torch::Tensor positions, torch::Tensor seq_len,
-                      c10::optional<torch::Tensor> r1,
-                      c10::optional<torch::Tensor> r2, double scale,
-                      double temp_coef, int64_t temp_every) {
-  const int T_ = out.size(0), H = out.size(1), dv = out.size(2);
-  const int G = kcache.size(1), ps = kcache.size(2), dk = kcache.size(3);
-  SEQ_CHECK(out.is_contiguous() && out.scalar_type() == proj.scalar_type(),
-            "attention out");
-  SEQ_CHECK(kcache.is_contiguous() && vcache.is_contiguous() &&
-                vcache.size(3) == dv && vcache.size(1) == G &&
-                kcache.scalar_type() == proj.scalar_type() &&
-                vcache.scalar_type() == proj.scalar_type(), "attention cache");
-  SEQ_CHECK(H % G == 0 && dv <= 64 * EVMAX, "attention head sizes");
-  SEQ_CHECK(proj.stride(1) == 1 && proj.size(0) == T_ &&
-                off_q + H * dk <= proj.size(1), "attention q");
+// out [T, H, kmaps, dv] (fp32 or the cache type); q rows in proj at off_q,
+// laid out [H][kmaps][dk]; kcache [P, G, ps, kmaps * dk]. Values come from
+// vcache [P, G, ps, dv], or - when vcache is absent - from the first dv
+// entries of each cached key row. window 0 = every earlier key is visible.
+void paged_attention_rows(torch::Tensor out, torch::Tensor proj, int64_t off_q,
+                          torch::Tensor kcache,
+                          c10::optional<torch::Tensor> vcache,
+                          torch::Tensor page_table, torch::Tensor tok_seq,
+                          torch::Tensor positions, torch::Tensor seq_len,
+                          c10::optional<torch::Tensor> r1,
+                          c10::optional<torch::Tensor> r2, double scale,
+                          double temp_coef, int64_t temp_every, int64_t kmaps,
+                          int64_t window) {
+  SEQ_CHECK(out.dim() == 4 && out.is_contiguous() && out.size(2) == kmaps,
+            "attention out [T, H, maps, dv]");
+  const int T_ = out.size(0), H = out.size(1), dv = out.size(3);
+  const int G = kcache.size(1), krow = kcache.size(3);
+  SEQ_CHECK(kmaps >= 1 && krow % kmaps == 0 && window >= 0, "key maps/window");
+  const int dk = krow / kmaps;
+  SEQ_CHECK(out.scalar_type() == proj.scalar_type() ||
+                out.scalar_type() == torch::kFloat, "attention out type");
+  SEQ_CHECK(kcache.is_contiguous() &&
+                kcache.scalar_type() == proj.scalar_type(), "attention cache");
+  const void* vptr;
+  int vrow;
+  if (vcache) {
+    SEQ_CHECK(vcache->is_contiguous() && vcache->size(3) == dv &&
+                  vcache->size(1) == G && vcache->size(2) == kcache.size(2) &&
+                  vcache->size(0) == kcache.size(0) &&
+                  vcache->scalar_type() == proj.scalar_type(),
+              "attention value cache");
+    vptr = vcache->data_ptr();
+    vrow = dv;
+  } else {
+    SEQ_CHECK(dv <= krow, "values inside the key rows");
+    vptr = kcache.data_ptr();
+    vrow = krow;
+  }
+  SEQ_CHECK(G >= 1 && H % G == 0 && dv >= 1 && dv <= 64 * EVMAX,
+            "attention head sizes");
+  SEQ_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(0) == T_ &&
+                off_q >= 0 && off_q + H * kmaps * dk <= proj.size(1),
+            "attention q");
   SEQ_CHECK(page_table.scalar_type() == torch::kInt && page_table.dim() == 2 &&
                 page_table.stride(1) == 1, "page table");
   for (const torch::Tensor* t : {&tok_seq, &positions})
@@ -415,12 +468,36 @@ void biased_attention(torch::Tensor out, torch::Tensor proj, int64_t off_q,
                 seq_len.numel() <= page_table.size(0), "seq_len");
   SEQ_CHECK(r1.has_value() == r2.has_value(), "bias parameters");
   if (r1)
-    SEQ_CHECK(r1->scalar_type() == torch::kFloat && r1->numel() == H &&
-                  r2->scalar_type() == torch::kFloat && r2->numel() == H,
-              "bias parameters");
+    SEQ_CHECK(kmaps == 1 && r1->scalar_type() == torch::kFloat &&
+                  r1->numel() == H && r2->scalar_type() == torch::kFloat &&
+                  r2->numel() == H, "bias parameters");
   SEQ_CHECK(temp_every >= 1, "temperature period");
   if (T_ == 0) return;
-  DISPATCH_ACT(proj, launch_attention<T>(
-      out, proj, off_q, kcache, vcache, page_table, tok_seq, positions,
-      seq_len, r1, r2, scale, temp_coef, temp_every););
+  const bool f32out = out.scalar_type() == torch::kFloat;
+  DISPATCH_ACT(proj, {
+    if (f32out)
+      launch_attention<T, float>(out, proj, off_q, kcache, vptr, dv, vrow,
+                                 page_table, tok_seq, positions, seq_len, r1,
+                                 r2, scale, temp_coef, temp_every, (int)kmaps,
+                                 (int)window);
+    else
+      launch_attention<T, T>(out, proj, off_q, kcache, vptr, dv, vrow,
+                             page_table, tok_seq, positions, seq_len, r1, r2,
+                             scale, temp_coef, temp_every, (int)kmaps,
+                             (int)window);
+  });
+}
+
+void biased_attention(torch::Tensor out, torch::Tensor proj, int64_t off_q,
+                      torch::Tensor kcache, torch::Tensor vcache,
+                      torch::Tensor page_table, torch::Tensor tok_seq,
+                      torch::Tensor positions, torch::Tensor seq_len,
+                      c10::optional<torch::Tensor> r1,
+                      c10::optional<torch::Tensor> r2, double scale,
+                      double temp_coef, int64_t temp_every) {
+  SEQ_CHECK(out.dim() == 3 && out.is_contiguous() &&
+                out.scalar_type() == proj.scalar_type(), "attention out");
+  paged_attention_rows(out.unsqueeze(2), proj, off_q, kcache, vcache,
+                       page_table, tok_seq, positions, seq_len, r1, r2, scale,
+                       temp_coef, temp_every, 1, 0);
 }

@@ -1,6 +1,6 @@
 // Python bindings for the sequence-mixer kernels (dynamo_amd._hip_seq):
-// recurrent matrix-state mixers, biased paged attention and their row-wise
-// companions. Built apart from dynamo_amd._hip so that a model which only
+// recurrent mixers (matrix-state and gated linear), paged attention over
+// rows (biased, windowed, multi-map, latent) and their row-wise companions. Built apart from dynamo_amd._hip so that a model which only
 // needs these compiles in seconds.
 #include <torch/extension.h>
 #include <pybind11/pybind11.h>
@@ -15,6 +15,9 @@ void add_scalar_rmsnorm(Tensor out, Tensor res, OptTensor delta, Tensor g,
 void causal_conv_silu(Tensor out, Tensor x, Tensor w, Tensor conv_state,
                       Tensor tok_seq, Tensor seq_start, Tensor seq_len,
                       Tensor seq_slot, Tensor seq_pos0);
+void causal_conv(Tensor out, Tensor x, Tensor w, OptTensor bias, bool silu,
+                 Tensor conv_state, Tensor tok_seq, Tensor seq_start,
+                 Tensor seq_len, Tensor seq_slot, Tensor seq_pos0);
 void token_shift_mix(Tensor out, Tensor h, Tensor mu, Tensor prev_state,
                      Tensor tok_seq, Tensor seq_start, Tensor seq_len,
                      Tensor seq_slot, Tensor seq_pos0);
@@ -44,6 +47,26 @@ void biased_attention(Tensor out, Tensor proj, int64_t off_q, Tensor kcache,
                       Tensor positions, Tensor seq_len, OptTensor r1,
                       OptTensor r2, double scale, double temp_coef,
                       int64_t temp_every);
+void paged_attention_rows(Tensor out, Tensor proj, int64_t off_q, Tensor kcache,
+                          OptTensor vcache, Tensor page_table, Tensor tok_seq,
+                          Tensor positions, Tensor seq_len, OptTensor r1,
+                          OptTensor r2, double scale, double temp_coef,
+                          int64_t temp_every, int64_t kmaps, int64_t window);
+void residual_layernorm(OptTensor out, Tensor res, OptTensor delta,
+                        OptTensor post_w, double mult, OptTensor w, double eps);
+void xielu(Tensor out, Tensor x, Tensor pq);
+void rope_rows(Tensor dst, int64_t dst_col, int64_t dst_vec, Tensor src,
+               int64_t src_col, int64_t src_vec, Tensor positions, Tensor freqs,
+               int64_t nvec, int64_t len, bool interleaved);
+void latent_append(Tensor cache, Tensor z, int64_t z_col, Tensor norm_w,
+                   Tensor slot_mapping, Tensor positions, Tensor freqs,
+                   bool interleaved, double eps);
+void diff_norm_gate(Tensor out, Tensor a, Tensor lambda, double post,
+                    OptTensor gate, double eps);
+void head_sigmoid_scale(Tensor out, Tensor x, Tensor gate);
+void rglru_scan(Tensor out, Tensor u, Tensor gates, Tensor br, Tensor bi,
+                Tensor lam, Tensor y, Tensor state, Tensor seq_start,
+                Tensor seq_len, Tensor seq_slot, Tensor seq_pos0, double decay);
 bool biased_attention_mfma_supported(int64_t dk, int64_t dv);
 void biased_attention_mfma(Tensor out, Tensor proj, int64_t off_q,
                            Tensor kcache, Tensor vcache, Tensor page_table,
@@ -57,6 +80,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("embed_scale_pos", &embed_scale_pos);
   m.def("add_scalar_rmsnorm", &add_scalar_rmsnorm);
   m.def("causal_conv_silu", &causal_conv_silu);
+  m.def("causal_conv", &causal_conv);
   m.def("token_shift_mix", &token_shift_mix);
   m.def("head_norm_gate", &head_norm_gate);
   m.def("clamped_glu", &clamped_glu);
@@ -67,6 +91,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("mlstm_memory", &mlstm_memory);
   m.def("kv_append_norm", &kv_append_norm);
   m.def("biased_attention", &biased_attention);
+  m.def("paged_attention_rows", &paged_attention_rows);
+  m.def("residual_layernorm", &residual_layernorm);
+  m.def("xielu", &xielu);
+  m.def("rope_rows", &rope_rows);
+  m.def("latent_append", &latent_append);
+  m.def("diff_norm_gate", &diff_norm_gate);
+  m.def("head_sigmoid_scale", &head_sigmoid_scale);
+  m.def("rglru_scan", &rglru_scan);
   m.def("biased_attention_mfma_supported", &biased_attention_mfma_supported);
   m.def("biased_attention_mfma", &biased_attention_mfma);
 }

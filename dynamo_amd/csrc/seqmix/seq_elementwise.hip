@@ -1,5 +1,6 @@
 // Row-wise kernels of the sequence-mixer models: embedding, scalar-gain RMS
-// norm fused with the fp32 residual add, short causal convolution, token
+// norm fused with the fp32 residual add, short causal convolution (with or
+// without bias and SiLU), token
 // shift, per-head output norm with gate, clamped GLU, two-branch merge and
 // the logit soft cap. All of them are bandwidth bound; one workgroup per
 // token row, fp32 arithmetic, activations in T.
@@ -50,13 +51,15 @@ __global__ void add_scalar_rmsnorm_kernel(T* __restrict__ out,
     out[(int64_t)t * W + i] = from_f<T>(r[i] * inv);
 }
 
-// y[t, c] = silu(sum_j w[c, j] * x[t - (taps-1) + j, c]); rows before the
-// start of this step's portion come from the slot's saved inputs (the last
-// taps-1 raw inputs of the sequence), or are zero at position 0.
+// y[t, c] = act(bias[c] + sum_j w[c, j] * x[t - (taps-1) + j, c]), act =
+// silu or identity, bias optional; rows before the start of this step's
+// portion come from the slot's saved inputs (the last taps-1 raw inputs of
+// the sequence), or are zero at position 0.
 template <typename T>
-__global__ void causal_conv_silu_kernel(
+__global__ void causal_conv_kernel(
     float* __restrict__ out, const T* __restrict__ x, int x_stride,
-    const float* __restrict__ w, const float* __restrict__ conv_state,
+    const float* __restrict__ w, const float* __restrict__ bias, int act,
+    const float* __restrict__ conv_state,
     const int* __restrict__ tok_seq, const int* __restrict__ seq_start,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_pos0,
     int C, int taps) {
@@ -66,7 +69,7 @@ __global__ void causal_conv_silu_kernel(
   const float* st = conv_state + (int64_t)seq_slot[s] * (taps - 1) * C;
   const int rel = t - start;  // rows of this portion before t
   for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float acc = 0.f;
+    float acc = bias ? bias[c] : 0.f;
     for (int j = 0; j < taps; j++) {
       const int back = taps - 1 - j;  // how many tokens before t
       float xv;
@@ -80,7 +83,7 @@ __global__ void causal_conv_silu_kernel(
       }
       acc += w[c * taps + j] * xv;
     }
-    out[(int64_t)t * C + c] = silu_f(acc);
+    out[(int64_t)t * C + c] = act ? silu_f(acc) : acc;
   }
 }
 
@@ -282,10 +285,11 @@ static void check_seq(const torch::Tensor& a, int64_t n, const char* what) {
                   a.numel() >= n, "seqmix: ", what, " must be int32 [>=", n, "]");
 }
 
-void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
-                      torch::Tensor conv_state, torch::Tensor tok_seq,
-                      torch::Tensor seq_start, torch::Tensor seq_len,
-                      torch::Tensor seq_slot, torch::Tensor seq_pos0) {
+void causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                 c10::optional<torch::Tensor> bias, bool silu,
+                 torch::Tensor conv_state, torch::Tensor tok_seq,
+                 torch::Tensor seq_start, torch::Tensor seq_len,
+                 torch::Tensor seq_slot, torch::Tensor seq_pos0) {
   // x: [T, >=C] rows of stride x.stride(0); the first C columns convolve
   const int T_ = x.size(0), C = w.size(0), taps = w.size(1);
   const int B = seq_start.size(0);
@@ -293,6 +297,9 @@ void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
   SEQ_CHECK(out.scalar_type() == torch::kFloat && out.is_contiguous() &&
                 out.size(0) == T_ && out.size(1) == C, "conv out");
   SEQ_CHECK(w.scalar_type() == torch::kFloat && w.is_contiguous(), "conv w");
+  if (bias)
+    SEQ_CHECK(bias->scalar_type() == torch::kFloat && bias->is_contiguous() &&
+                  bias->numel() == C, "conv bias");
   SEQ_CHECK(conv_state.scalar_type() == torch::kFloat &&
                 conv_state.is_contiguous() && conv_state.size(1) == taps - 1 &&
                 conv_state.size(2) == C, "conv state");
@@ -302,10 +309,12 @@ void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
   check_seq(seq_pos0, B, "seq_pos0");
   if (T_ == 0) return;
   DISPATCH_ACT(x, {
-    hipLaunchKernelGGL(causal_conv_silu_kernel<T>, dim3(T_), dim3(row_block(C)),
+    hipLaunchKernelGGL(causal_conv_kernel<T>, dim3(T_), dim3(row_block(C)),
                        0, cur_stream(), ptr<float>(out), cptr<T>(x),
                        (int)x.stride(0), cptr<float>(w),
-                       cptr<float>(conv_state), cptr<int>(tok_seq),
+                       bias ? cptr<float>(*bias) : (const float*)nullptr,
+                       silu ? 1 : 0, cptr<float>(conv_state),
+                       cptr<int>(tok_seq),
                        cptr<int>(seq_start), cptr<int>(seq_slot),
                        cptr<int>(seq_pos0), C, taps);
     if (taps > 1)
@@ -315,6 +324,14 @@ void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
                          cptr<int>(seq_start), cptr<int>(seq_len),
                          cptr<int>(seq_slot), cptr<int>(seq_pos0), C, taps);
   });
+}
+
+void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                      torch::Tensor conv_state, torch::Tensor tok_seq,
+                      torch::Tensor seq_start, torch::Tensor seq_len,
+                      torch::Tensor seq_slot, torch::Tensor seq_pos0) {
+  causal_conv(out, x, w, c10::nullopt, true, conv_state, tok_seq, seq_start,
+              seq_len, seq_slot, seq_pos0);
 }
 
 void token_shift_mix(torch::Tensor out, torch::Tensor h, torch::Tensor mu,

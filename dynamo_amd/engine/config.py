@@ -16,7 +16,7 @@ from typing import Optional
 @dataclass
 class ModelConfig:
     name: str = "llama-3-8b"
-    arch: str = "llama"            # llama | opt | mixtral | qwen2 | bolatar
+    arch: str = "llama"            # llama | opt | mixtral | qwen2 | bolatar | fironex
     hidden_size: int = 4096
     intermediate_size: int = 14336
     num_layers: int = 32
@@ -39,11 +39,12 @@ class ModelConfig:
     learned_pos_emb: bool = False
     # qwen2-style QKV bias
     attn_bias: bool = False
-    # layer-list models (bolatar): one dict per layer with its mixer type,
+    # layer-list models (bolatar, fironex): one dict per layer with its mixer type,
     # mixer sizes and feed-forward, as in the checkpoint's config.json
     layer_specs: Optional[list] = None
     embed_scale: float = 1.0       # multiplies token embeddings
     logit_softcap: float = 0.0     # cap * tanh(logits / cap); 0 = off
+    residual_mult: float = 1.0     # scales a normed sublayer output (fironex)
     # local HF checkpoint dir to load real weights from ("" = random init)
     weights_path: str = ""
 
@@ -133,6 +134,34 @@ PRESETS = {
             {"type": "mlstm", "mixer": {"heads": 2, "dim": 16, "vdim": 48,
                                         "gate_cap": 10.0},
              "mlp": {"kind": "dense", "ff": 120, "limit": 2.5}},
+        ]),
+    # layer-list model with layer norms around every sublayer: every mixer
+    # kind once (the second latent layer reads the first one's cache)
+    "tiny-fironex": ModelConfig(
+        name="tiny-fironex", arch="fironex", hidden_size=96, vocab_size=160,
+        num_layers=4, rms_eps=1e-5, residual_mult=0.8, tie_embeddings=True,
+        norm="layernorm", intermediate_size=0, num_q_heads=1, num_kv_heads=1,
+        head_dim=1,
+        layer_specs=[
+            {"type": "latent_attention", "mixer": {
+                "heads": 3, "dim": 24, "rot_dim": 8, "vdim": 20,
+                "kv_rank": 40, "scale": 0.18,
+                "rot": {"base": 5000.0, "dims": 8}},
+             "mlp": {"kind": "dense", "ff": 144}},
+            {"type": "rglru", "mixer": {"width": 72, "blocks": 3, "conv": 3},
+             "mlp": None},
+            {"type": "latent_attention", "mixer": {
+                "heads": 2, "dim": 16, "rot_dim": 8, "vdim": 28,
+                "kv_rank": 40, "scale": 0.2, "kv_from": 0,
+                "rot": {"base": 5000.0, "dims": 8}},
+             "mlp": {"kind": "dense", "ff": 120}},
+            {"type": "attention", "mixer": {
+                "heads": 6, "kv_heads": 3, "dim": 24, "vdim": 40,
+                "scale": 0.2, "diff": 0.3, "mask": {"size": 24},
+                "rot": {"base": 10000.0, "dims": 12,
+                        "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0,
+                                    "original": 64}}},
+             "mlp": {"kind": "dense", "ff": 100}},
         ]),
 }
 

@@ -39,9 +39,13 @@ def config_from_hf(path: str) -> ModelConfig:
     """Build a ModelConfig from an HF checkpoint dir's config.json."""
     with open(os.path.join(path, "config.json")) as f:
         hf = json.load(f)
-    if str(hf.get("architecture", "")).lower() == "bolatar":
-        from dynamo_amd.models.bolatar import config_from_json
-        return config_from_json(hf, os.path.basename(os.path.normpath(path)))
+    from dynamo_amd.models.registry import LAYER_LIST_ARCHS
+    kind = str(hf.get("architecture", "")).lower()
+    if kind in LAYER_LIST_ARCHS:
+        import importlib
+        reader = importlib.import_module(LAYER_LIST_ARCHS[kind])
+        return reader.config_from_json(
+            hf, os.path.basename(os.path.normpath(path)))
     archs = [a.lower() for a in hf.get("architectures", [])]
     if any("mixtral" in a for a in archs):
         arch = "mixtral"

@@ -1,6 +1,8 @@
-"""Token mixers beyond rotary softmax attention: recurrent matrix-state
-mixers with a slot-addressed fp32 state, and softmax attention with a
-distance bias / query temperature / value norm over the paged cache.
+"""Token mixers beyond rotary softmax attention: recurrent mixers with a
+slot-addressed fp32 state (matrix memories, a gated linear unit), and
+softmax attention over the paged cache with a distance bias / query
+temperature / value norm, with differential heads under a sliding window,
+or over a shared compressed latent.
 
 Every mixer takes the normed hidden rows h [T, W] of the engine's flat
 batch and a `MixContext` (sequence spans, state tensors of its layer, cache
@@ -320,3 +322,242 @@ class ClampedGLU(torch.nn.Module):
         act = sops.clamped_glu(F.linear(h, self.w_gate_up), self.limit,
                                self.alpha)
         return F.linear(act, self.w_down)
+
+
+def rotary_frequencies(rot: dict) -> torch.Tensor:
+    """fp32 [dims/2] angular frequencies base^(-2i/dims) of a rotary spec
+    {"base", "dims", "scaling"?}. The optional scaling {factor, low, high,
+    original} slows long wavelengths (above original/low) by `factor`,
+    keeps short ones (below original/high) and blends linearly in between.
+    Evaluated in float64, stored in fp32; angles are position * frequency
+    in fp32 inside the kernels."""
+    import math
+    n = int(rot["dims"])
+    f = [float(rot["base"]) ** (-2.0 * i / n) for i in range(n // 2)]
+    sc = rot.get("scaling")
+    if sc:
+        lo_wl = sc["original"] / sc["high"]
+        hi_wl = sc["original"] / sc["low"]
+        for i, fi in enumerate(f):
+            wl = 2 * math.pi / fi
+            if wl > hi_wl:
+                f[i] = fi / sc["factor"]
+            elif wl >= lo_wl:
+                s = (sc["original"] / wl - sc["low"]) / (sc["high"] - sc["low"])
+                f[i] = (1 - s) * fi / sc["factor"] + s * fi
+    return torch.tensor(f, dtype=torch.float64).to(torch.float32)
+
+
+class RGLRUMixer(torch.nn.Module):
+    """Recurrent block around a real-gated linear recurrent unit: a gate
+    branch gelu_tanh(W_y h + b_y) beside u = conv(W_x h + b_x) (short causal
+    per-channel convolution with bias, no activation). Per channel, with
+    block-diagonal gate matrices over `blocks` equal parts of u:
+      r = sigmoid(A_r u + b_r), i = sigmoid(A_i u + b_i),
+      a = exp(-decay r softplus(lam)), S <- a S + sqrt(1 - a^2) i u.
+    Output W_o (S * gate branch). Gates and the recurrence run in fp32."""
+
+    def __init__(self, width, channels, blocks, conv, init, decay=8.0):
+        super().__init__()
+        if channels % blocks:
+            raise ValueError("recurrence width must divide into its blocks")
+        self.W, self.C, self.nb, self.taps = width, channels, blocks, conv
+        self.bw = channels // blocks
+        self.decay = decay
+        f32 = dict(dtype=torch.float32, device=init.device)
+        # fused rows: x (convolved) | y (gate branch)
+        self.w_in = init.mat(2 * channels, width)
+        self.b_in = init.vec(2 * channels, -0.2, 0.2).to(init.dtype)
+        self.conv_w = init.vec((channels, conv), -0.5, 0.8)
+        self.conv_b = init.vec(channels, -0.2, 0.2)
+        # gate matrices as x @ w per block: [nb, bw(in), 2 bw (r | i)]
+        self.w_gates = (torch.randn(blocks, self.bw, 2 * self.bw,
+                                    generator=init.gen) * self.bw ** -0.5
+                        ).to(**f32)
+        self.b_r = init.vec(channels, -0.5, 0.5)
+        self.b_i = init.vec(channels, -0.5, 0.5)
+        self.lam = init.vec(channels, -4.0, -1.0)
+        self.w_o = init.mat(width, channels)
+
+    def state_shapes(self):
+        return [(self.C,), (self.taps - 1, self.C)]
+
+    def kv_shape(self):
+        return None
+
+    def load(self, get: Getter):
+        _put(self.w_in, torch.cat([get("x"), get("y")], 0))
+        _put(self.b_in, torch.cat([get("x.b"), get("y.b")], 0))
+        _put(self.conv_w, get("conv"))
+        _put(self.conv_b, get("conv.b"))
+        # checkpoint matrices are [block, out, in]
+        _put(self.w_gates, torch.cat([get("ra").transpose(1, 2),
+                                      get("ri").transpose(1, 2)], 2))
+        _put(self.b_r, get("ra.b").reshape(-1))
+        _put(self.b_i, get("ri.b").reshape(-1))
+        _put(self.lam, get("lam"))
+        _put(self.w_o, get("o"))
+
+    def forward(self, h, ctx: MixContext):
+        T = h.shape[0]
+        proj = F.linear(h, self.w_in, self.b_in)
+        S, conv_state = ctx.states
+        u = sops.causal_conv(proj, self.C, self.conv_w, self.conv_b, False,
+                             conv_state, ctx.sb)
+        gates = torch.bmm(u.view(T, self.nb, self.bw).transpose(0, 1),
+                          self.w_gates)
+        y = sops.rglru_scan(u, gates, self.b_r, self.b_i, self.lam,
+                            proj[:, self.C:], S, ctx.sb, self.decay, h.dtype)
+        return F.linear(y, self.w_o)
+
+
+class DifferentialAttention(torch.nn.Module):
+    """Grouped-query attention whose heads each run two softmax maps over
+    the same values and subtract them: o = a1 - lam a2, then a weightless
+    RMS norm per head times (1 - diff) and an element-wise sigmoid output
+    gate. lam = exp(lq1 . lk1) - exp(lq2 . lk2) + diff for the whole layer.
+    Queries/keys of both maps are rotated (interleaved pairs, first
+    rot.dims entries); an optional sliding window bounds the visible keys.
+    The paged cache row of a kv head holds both maps' keys back to back."""
+
+    def __init__(self, width, heads, kv_heads, dim, vdim, scale, diff, rot,
+                 window, eps, init):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("query heads must be a multiple of kv heads")
+        self.W, self.H, self.G, self.dk, self.dv = width, heads, kv_heads, dim, vdim
+        self.scale, self.diff, self.eps = scale, diff, eps
+        self.window = int(window or 0)
+        self.off_k = heads * 2 * dim
+        self.off_v = self.off_k + kv_heads * 2 * dim
+        self.off_g = self.off_v + kv_heads * vdim
+        # fused rows: q | k | v | gate
+        self.w_in = init.mat(self.off_g + heads * vdim, width)
+        self.freqs = rotary_frequencies(rot).to(init.device)
+        if 2 * self.freqs.numel() > dim:
+            raise ValueError("rotary dims exceed the head size")
+        self.lq1, self.lk1 = init.vec(dim, -0.3, 0.3), init.vec(dim, -0.3, 0.3)
+        self.lq2, self.lk2 = init.vec(dim, -0.3, 0.3), init.vec(dim, -0.3, 0.3)
+        self.w_o = init.mat(width, heads * vdim)
+        self.refresh()
+
+    def refresh(self):
+        """The layer's lambda from its four vectors (fp32)."""
+        self.lam = (torch.exp((self.lq1 * self.lk1).sum())
+                    - torch.exp((self.lq2 * self.lk2).sum())
+                    + self.diff).reshape(1).float()
+
+    def state_shapes(self):
+        return []
+
+    def kv_shape(self):
+        return (self.G, 2 * self.dk, self.dv)
+
+    def load(self, get: Getter):
+        _put(self.w_in, torch.cat([get("q"), get("k"), get("v"), get("g")], 0))
+        for n in ("lq1", "lk1", "lq2", "lk2"):
+            _put(getattr(self, n), get(n))
+        _put(self.w_o, get("o"))
+        self.refresh()
+
+    def forward(self, h, ctx: MixContext):
+        proj = F.linear(h, self.w_in)
+        # q and k of both maps are 2H + 2G vectors of dk, back to back
+        sops.rope_rows(proj, 0, self.dk, proj, 0, self.dk, ctx.positions,
+                       self.freqs, 2 * (self.H + self.G), self.dk, True)
+        sops.kv_append_norm(ctx.kcache, ctx.vcache, proj, self.off_k,
+                            self.off_v, ctx.slot_mapping, False, self.eps)
+        a = sops.paged_attention_rows(proj, 0, self.H, 2, ctx.kcache,
+                                      ctx.vcache, self.dv, ctx.positions,
+                                      ctx.sb, self.scale, self.window)
+        y = sops.diff_norm_gate(a, self.lam, 1.0 - self.diff,
+                                proj[:, self.off_g:], self.eps, h.dtype)
+        return F.linear(y, self.w_o)
+
+
+class LatentAttention(torch.nn.Module):
+    """Causal attention over a compressed cache: per token only an
+    RMS-normed latent c [rank] and one rotated key part [rot_dim] shared by
+    all heads are stored. Head keys W_uk c and values W_uv c are never
+    materialised: W_uk is folded into the query and W_uv applied to the
+    attention-weighted latent, so the kernel runs as multi-query attention
+    whose values are the first `rank` entries of the cached rows. Rotation
+    pairs (i, i + dims/2) over the rot_dim part; per-head sigmoid output
+    gate. With shared_cache the layer has no down-projection of its own and
+    reads another latent layer's cache."""
+
+    def __init__(self, width, heads, dim, rot_dim, vdim, rank, scale, rot, eps,
+                 init, shared_cache=False):
+        super().__init__()
+        self.W, self.H, self.dk, self.rd, self.dv = width, heads, dim, rot_dim, vdim
+        self.rank, self.scale, self.eps = rank, scale, eps
+        self.shared_cache = shared_cache
+        self.freqs = rotary_frequencies(rot).to(init.device)
+        if 2 * self.freqs.numel() > rot_dim:
+            raise ValueError("rotary dims exceed the rotated part")
+        self.off_z = heads * (dim + rot_dim)
+        self.off_g = self.off_z + (0 if shared_cache else rank + rot_dim)
+        # fused rows: q | [latent down-projection] | gate
+        self.w_in = init.mat(self.off_g + heads, width)
+        self.dkv_norm = None if shared_cache else init.vec(rank, 0.7, 1.3)
+        self.w_uk = torch.stack([init.mat(dim, rank) for _ in range(heads)])
+        self.w_uv_t = torch.stack([init.mat(vdim, rank).t().contiguous()
+                                   for _ in range(heads)])
+        self.w_o = init.mat(width, heads * vdim)
+
+    def state_shapes(self):
+        return []
+
+    def kv_shape(self):
+        return None if self.shared_cache else (1, self.rank + self.rd, 0)
+
+    def load(self, get: Getter):
+        rows = [get("q")] + ([] if self.shared_cache else [get("dkv")])
+        _put(self.w_in, torch.cat(rows + [get("g")], 0))
+        if not self.shared_cache:
+            _put(self.dkv_norm, get("dkv.norm"))
+        _put(self.w_uk, get("uk").view(self.H, self.dk, self.rank))
+        _put(self.w_uv_t, get("uv").view(self.H, self.dv,
+                                         self.rank).transpose(1, 2))
+        _put(self.w_o, get("o"))
+
+    def forward(self, h, ctx: MixContext):
+        T, H, R, rd = h.shape[0], self.H, self.rank, self.rd
+        proj = F.linear(h, self.w_in)
+        if not self.shared_cache:
+            sops.latent_append(ctx.kcache, proj, self.off_z, self.dkv_norm,
+                               ctx.slot_mapping, ctx.positions, self.freqs,
+                               False, self.eps)
+        qh = proj[:, :self.off_z].view(T, H, self.dk + rd)
+        q = torch.empty(T, H * (R + rd), dtype=h.dtype, device=h.device)
+        q.view(T, H, R + rd)[:, :, :R].copy_(
+            torch.bmm(qh[:, :, :self.dk].transpose(0, 1),
+                      self.w_uk).transpose(0, 1))
+        sops.rope_rows(q, R, R + rd, proj, self.dk, self.dk + rd,
+                       ctx.positions, self.freqs, H, rd, False)
+        lat = sops.paged_attention_rows(q, 0, H, 1, ctx.kcache, None, R,
+                                        ctx.positions, ctx.sb, self.scale, 0)
+        g = sops.head_sigmoid_scale(lat.view(T, H, R), proj[:, self.off_g:],
+                                    h.dtype)
+        o = torch.bmm(g, self.w_uv_t)                       # [H, T, dv]
+        return F.linear(o.transpose(0, 1).reshape(T, H * self.dv), self.w_o)
+
+
+class XIELUMLP(torch.nn.Module):
+    """Dense feed-forward W_down xIELU(W_up h) with the activation's two raw
+    parameters (softplus-ed inside the kernel)."""
+
+    def __init__(self, width, ff, init):
+        super().__init__()
+        self.w_up = init.mat(ff, width)
+        self.w_down = init.mat(width, ff)
+        self.act = init.vec(2, -1.0, 1.0)
+
+    def load(self, get: Getter):
+        _put(self.w_up, get("up"))
+        _put(self.w_down, get("down"))
+        _put(self.act, get("act"))
+
+    def forward(self, h):
+        return F.linear(sops.xielu(F.linear(h, self.w_up), self.act),
+                        self.w_down)

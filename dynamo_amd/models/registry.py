@@ -17,7 +17,24 @@ def build_model(cfg: ModelConfig, device, dtype, tp=None, seed: int = 0):
     if cfg.arch == "bolatar":
         from .bolatar import BolatarForCausalLM
         return BolatarForCausalLM(cfg, device, dtype, tp, seed)
+    if cfg.arch == "fironex":
+        from .fironex import FironexForCausalLM
+        return FironexForCausalLM(cfg, device, dtype, tp, seed)
     raise ValueError(f"unknown arch {cfg.arch}")
+
+
+# config.json "architecture" values of layer-list checkpoints -> the module
+# whose config_from_json reads them
+LAYER_LIST_ARCHS = {"bolatar": "dynamo_amd.models.bolatar",
+                    "fironex": "dynamo_amd.models.fironex"}
+
+
+def native_extensions(cfg: ModelConfig, device: str):
+    """Names of the in-tree extensions a model needs on `device`."""
+    exts = ["_core"]
+    if str(device).startswith("cuda"):
+        exts.append("_hip_seq" if cfg.arch in LAYER_LIST_ARCHS else "_hip")
+    return exts
 
 
 def resolve_model_config(name_or_cfg) -> ModelConfig:

@@ -233,3 +233,123 @@ def biased_attention(proj, off_q: int, H: int, kcache, vcache, positions,
         return out.view(T, H * dv)
     return seq_ref.biased_attention(proj, off_q, H, kcache, vcache, positions,
                                     sb, r1, r2, scale, temp_coef, temp_every)
+
+
+# -- layer-norm sandwiched layers ----------------------------------------------
+def residual_layernorm(res, delta, post_w, mult: float, w, eps: float,
+                       out_dtype):
+    """res (fp32, in place) += mult * LN(delta) * post_w when delta is given
+    (plain += delta without post_w); returns LN(res) * w in out_dtype, or
+    None when w is None. LN is the weight-only layer norm."""
+    if res.is_cuda:
+        out = (torch.empty(res.shape, dtype=out_dtype, device=res.device)
+               if w is not None else None)
+        hip_seq().residual_layernorm(out, res, delta, post_w, float(mult), w,
+                                     float(eps))
+        return out
+    return seq_ref.residual_layernorm(res, delta, post_w, mult, w, eps,
+                                      out_dtype)
+
+
+def xielu(x, pq):
+    """xIELU with raw parameters pq = (p, q): softplus(p) z^2 + z/2 for
+    z > 0, (1/2 + softplus(q)) (e^z - 1 - z) + z/2 otherwise."""
+    if x.is_cuda:
+        out = torch.empty_like(x)
+        hip_seq().xielu(out, x, pq)
+        return out
+    return seq_ref.xielu(x, pq)
+
+
+def rope_rows(dst, dst_col: int, dst_vec: int, src, src_col: int,
+              src_vec: int, positions, freqs, nvec: int, length: int,
+              interleaved: bool):
+    """For each token row, `nvec` vectors of `length` entries (vector v at
+    column col + v * vec) go from src to dst with their first
+    2 * len(freqs) entries rotated by position * freqs; dst may be src."""
+    if src.is_cuda:
+        hip_seq().rope_rows(dst, dst_col, dst_vec, src, src_col, src_vec,
+                            positions, freqs, nvec, length, bool(interleaved))
+    else:
+        seq_ref.rope_rows(dst, dst_col, dst_vec, src, src_col, src_vec,
+                          positions, freqs, nvec, length, interleaved)
+
+
+def latent_append(cache, z, z_col: int, norm_w, slot_mapping, positions,
+                  freqs, interleaved: bool, eps: float):
+    """cache [P, 1, ps, rank + rd] <- [rmsnorm(z[:rank]) * norm_w |
+    rotated z[rank:rank + rd]] at each token's slot."""
+    if z.is_cuda:
+        hip_seq().latent_append(cache, z, z_col, norm_w, slot_mapping,
+                                positions, freqs, bool(interleaved),
+                                float(eps))
+    else:
+        seq_ref.latent_append(cache, z, z_col, norm_w, slot_mapping,
+                              positions, freqs, interleaved, eps)
+
+
+def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
+                         dv: int, positions, sb: SeqBatch, scale: float,
+                         window: int = 0):
+    """Causal softmax attention of every row over its sequence's pages.
+    -> fp32 [T, H, kmaps, dv]. Queries lie in q at off_q as [H][kmaps][dk];
+    kcache [P, G, ps, kmaps * dk]; values from vcache [P, G, ps, dv] or,
+    without one, from the first dv entries of the key rows. window > 0:
+    row i sees keys j with 0 <= i - j < window."""
+    if q.is_cuda:
+        T = q.shape[0]
+        out = torch.empty(T, H, kmaps, dv, dtype=torch.float32,
+                          device=q.device)
+        hip_seq().paged_attention_rows(
+            out, q, off_q, kcache, vcache, sb.page_table, sb.tok_seq,
+            positions, sb.seq_len, None, None, float(scale), 0.0, 1,
+            int(kmaps), int(window))
+        return out
+    return seq_ref.paged_attention_rows(q, off_q, H, kmaps, kcache, vcache,
+                                        dv, positions, sb, scale, window)
+
+
+def diff_norm_gate(a, lam, post: float, gate, eps: float, out_dtype):
+    """a fp32 [T, H, 2, dv] -> [T, H*dv]: (a1 - lam a2) / rms * post *
+    sigmoid(gate)."""
+    if a.is_cuda:
+        T, H, _two, dv = a.shape
+        out = torch.empty(T, H * dv, dtype=out_dtype, device=a.device)
+        hip_seq().diff_norm_gate(out, a, lam, float(post), gate, float(eps))
+        return out
+    return seq_ref.diff_norm_gate(a, lam, post, gate, eps, out_dtype)
+
+
+def head_sigmoid_scale(x, gate, out_dtype):
+    """x fp32 [T, H, R], gate [T, >=H] -> [H, T, R] = x * sigmoid(gate)."""
+    if x.is_cuda:
+        T, H, R = x.shape
+        out = torch.empty(H, T, R, dtype=out_dtype, device=x.device)
+        hip_seq().head_sigmoid_scale(out, x, gate)
+        return out
+    return seq_ref.head_sigmoid_scale(x, gate, out_dtype)
+
+
+def causal_conv(x, C: int, w, bias, silu: bool, conv_state, sb: SeqBatch):
+    """Short causal convolution over the first C columns of x with optional
+    bias and SiLU; fp32 out. The slot's saved inputs continue earlier
+    portions and are updated."""
+    if x.is_cuda:
+        out = torch.empty(x.shape[0], C, dtype=torch.float32, device=x.device)
+        hip_seq().causal_conv(out, x, w, bias, bool(silu), conv_state,
+                              sb.tok_seq, *_args(sb))
+        return out
+    return seq_ref.causal_conv(x, C, w, bias, silu, conv_state, sb)
+
+
+def rglru_scan(u, gates, br, bi, lam, y, state, sb: SeqBatch, decay: float,
+               out_dtype):
+    """Real-gated linear recurrence over fp32 u [T, C] with gate
+    pre-activations gates [nb, T, 2*bw]; returns S * gelu_tanh(y[:, :C])."""
+    if u.is_cuda:
+        out = torch.empty(u.shape, dtype=out_dtype, device=u.device)
+        hip_seq().rglru_scan(out, u, gates, br, bi, lam, y, state, *_args(sb),
+                             float(decay))
+        return out
+    return seq_ref.rglru_scan(u, gates, br, bi, lam, y, state, sb, decay,
+                              out_dtype)

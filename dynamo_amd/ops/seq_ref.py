@@ -229,3 +229,168 @@ def biased_attention(proj, off_q, H, kcache, vcache, positions, sb, r1, r2,
             out[t] = torch.einsum("hj,hjd->hd", torch.softmax(s, -1),
                                   vv[:, :i + 1])
     return out.to(proj.dtype).view(T, H * dv)
+
+
+# -- layer-norm sandwiched layers, rotary, differential / latent attention -----
+def _ln(x, w, eps):
+    mu = x.mean(-1, keepdim=True)
+    var = (x - mu).pow(2).mean(-1, keepdim=True)
+    return (x - mu) / torch.sqrt(var + eps) * w
+
+
+def residual_layernorm(res, delta, post_w, mult, w, eps, out_dtype):
+    if delta is not None:
+        d = delta.float()
+        res.add_(mult * _ln(d, post_w, eps) if post_w is not None else d)
+    if w is None:
+        return None
+    return _ln(res, w, eps).to(out_dtype)
+
+
+def xielu(x, pq):
+    z = x.float()
+    ap, aq = F.softplus(pq[0]), 0.5 + F.softplus(pq[1])
+    y = torch.where(z > 0, ap * z * z + 0.5 * z,
+                    aq * (torch.expm1(z.clamp(max=0)) - z) + 0.5 * z)
+    return y.to(x.dtype)
+
+
+def _rotate(x, positions, freqs, interleaved):
+    """x fp32 [T, n, len]; the first 2 * len(freqs) entries are rotated."""
+    dims = 2 * freqs.numel()
+    ang = positions.float()[:, None] * freqs[None, :]
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    y = x.clone()
+    if interleaved:
+        a, b = x[..., 0:dims:2], x[..., 1:dims:2]
+        y[..., 0:dims:2] = a * c - b * s
+        y[..., 1:dims:2] = b * c + a * s
+    else:
+        h = dims // 2
+        a, b = x[..., :h], x[..., h:dims]
+        y[..., :h] = a * c - b * s
+        y[..., h:dims] = b * c + a * s
+    return y
+
+
+def rope_rows(dst, dst_col, dst_vec, src, src_col, src_vec, positions, freqs,
+              nvec, length, interleaved):
+    T = src.shape[0]
+    if T == 0 or nvec == 0:
+        return
+    x = torch.stack([src[:, src_col + v * src_vec:src_col + v * src_vec + length]
+                     for v in range(nvec)], 1).float()
+    y = _rotate(x, positions, freqs, interleaved).to(dst.dtype)
+    for v in range(nvec):
+        dst[:, dst_col + v * dst_vec:dst_col + v * dst_vec + length] = y[:, v]
+
+
+def latent_append(cache, z, z_col, norm_w, slot_mapping, positions, freqs,
+                  interleaved, eps):
+    P, _one, ps, row = cache.shape
+    rank = norm_w.numel()
+    zz = z[:, z_col:z_col + row].float()
+    c = zz[:, :rank]
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_w
+    kr = _rotate(zz[:, None, rank:], positions, freqs, interleaved)[:, 0]
+    rows = torch.cat([c, kr], -1).to(cache.dtype)
+    for t, slot in enumerate(slot_mapping.tolist()):
+        if slot >= 0:
+            cache[slot // ps, 0, slot % ps] = rows[t]
+
+
+def paged_attention_rows(q, off_q, H, kmaps, kcache, vcache, dv, positions, sb,
+                         scale, window):
+    """fp32 [T, H, kmaps, dv]; see ops.seq.paged_attention_rows."""
+    P, G, ps, krow = kcache.shape
+    dk = krow // kmaps
+    T = q.shape[0]
+    qq = q[:, off_q:off_q + H * kmaps * dk].float().view(T, H, kmaps, dk)
+    out = torch.zeros(T, H, kmaps, dv, dtype=torch.float32)
+    pos = positions.tolist()
+    rep = H // G
+    for si, (start, n, slot, pos0) in enumerate(sb.spans()):
+        if n == 0:
+            continue
+        pages = sb.page_table[si].long()
+        ctx = pos0 + n
+        npg = (ctx + ps - 1) // ps
+        kk = kcache[pages[:npg]].float().permute(1, 0, 2, 3).reshape(
+            G, npg * ps, kmaps, dk)[:, :ctx]
+        if vcache is not None:
+            vv = vcache[pages[:npg]].float().permute(1, 0, 2, 3).reshape(
+                G, npg * ps, dv)[:, :ctx]
+        else:
+            vv = kk.reshape(G, ctx, krow)[:, :, :dv]
+        kk = kk.repeat_interleave(rep, 0)
+        vv = vv.repeat_interleave(rep, 0)
+        for t in range(start, start + n):
+            i = pos[t]
+            lo = max(0, i + 1 - window) if window else 0
+            s = torch.einsum("hmd,hjmd->hmj", qq[t] * scale, kk[:, lo:i + 1])
+            out[t] = torch.einsum("hmj,hjd->hmd", torch.softmax(s, -1),
+                                  vv[:, lo:i + 1])
+    return out
+
+
+def diff_norm_gate(a, lam, post, gate, eps, out_dtype):
+    T, H, _two, dv = a.shape
+    o = a[:, :, 0] - lam.reshape(()) * a[:, :, 1]
+    o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * post
+    if gate is not None:
+        o = o * torch.sigmoid(gate[:, :H * dv].float().view(T, H, dv))
+    return o.reshape(T, H * dv).to(out_dtype)
+
+
+def head_sigmoid_scale(x, gate, out_dtype):
+    T, H, R = x.shape
+    g = torch.sigmoid(gate[:, :H].float())
+    return (x * g[:, :, None]).transpose(0, 1).contiguous().to(out_dtype)
+
+
+def causal_conv(x, C, w, bias, silu, conv_state, sb):
+    taps = w.shape[1]
+    K = taps - 1
+    xin = x[:, :C].float()
+    out = torch.empty(x.shape[0], C, dtype=torch.float32)
+    for start, n, slot, pos0 in sb.spans():
+        if n == 0:
+            continue
+        hist = (conv_state[slot].clone() if pos0 > 0
+                else torch.zeros(K, C, dtype=torch.float32))
+        if 0 < pos0 < K:
+            hist[:K - pos0] = 0
+        full = torch.cat([hist, xin[start:start + n]], 0)
+        acc = torch.zeros(n, C, dtype=torch.float32)
+        if bias is not None:
+            acc += bias
+        for j in range(taps):
+            acc += full[j:j + n] * w[:, j]
+        out[start:start + n] = F.silu(acc) if silu else acc
+        if K:
+            conv_state[slot] = full[-K:]
+    return out
+
+
+def rglru_scan(u, gates, br, bi, lam, y, state, sb, decay, out_dtype):
+    T, C = u.shape
+    nb, _t, two_bw = gates.shape
+    bw = two_bw // 2
+    gr = gates[:, :, :bw].permute(1, 0, 2).reshape(T, C)
+    gi = gates[:, :, bw:].permute(1, 0, 2).reshape(T, C)
+    r = torch.sigmoid(gr + br)
+    ig = torch.sigmoid(gi + bi)
+    la = -decay * F.softplus(lam) * r
+    a = torch.exp(la)
+    b = torch.sqrt(-torch.expm1(2 * la)) * (ig * u)
+    yy = F.gelu(y[:, :C].float(), approximate="tanh")
+    out = torch.empty(T, C, dtype=torch.float32)
+    for start, n, slot, pos0 in sb.spans():
+        if n == 0:
+            continue
+        S = state[slot].clone() if pos0 > 0 else torch.zeros(C)
+        for t in range(start, start + n):
+            S = a[t] * S + b[t]
+            out[t] = S * yy[t]
+        state[slot] = S
+    return out.to(out_dtype)

@@ -75,16 +75,14 @@ def main(argv=None) -> int:
                     help="sequences that may be live at once")
     a = ap.parse_args(argv)
 
-    with open(os.path.join(a.model, "config.json")) as f:
-        is_seq = str(json.load(f).get("architecture", "")).lower() == "bolatar"
     import torch
     device = a.device
     if device == "auto":
         device = "cuda:0" if torch.cuda.is_available() else "cpu"
-    exts = ["_core"]
-    if device.startswith("cuda"):
-        exts.append("_hip_seq" if is_seq else "_hip")
-    ensure_built(exts)
+    from dynamo_amd.models.registry import (native_extensions,
+                                            resolve_model_config)
+    model = resolve_model_config(a.model)
+    ensure_built(native_extensions(model, device))
 
     if a.dtype == "float32":
         torch.backends.cuda.matmul.allow_tf32 = False
@@ -92,8 +90,6 @@ def main(argv=None) -> int:
         torch.set_float32_matmul_precision("highest")
 
     from dynamo_amd.engine import EngineConfig, LLMEngine
-    from dynamo_amd.models.registry import resolve_model_config
-    model = resolve_model_config(a.model)
     page = 64
     cfg = EngineConfig(
         model=model, device=device, dtype=a.dtype, page_size=page,
