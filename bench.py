@@ -55,8 +55,13 @@ def parse_args():
     p.add_argument("--max-batched-tokens", type=int, default=0)
     p.add_argument("--mixer-compare", action="store_true",
                    help="instead of the flagship workload: prefill/decode "
-                        "throughput of the layer-list (Bolatar) design "
-                        "beside Llama at equal sizes (1 GPU)")
+                        "throughput of a layer-list design (see "
+                        "--mixer-model) beside Llama at equal sizes (1 GPU)")
+    p.add_argument("--mixer-model", default="bolatar",
+                   choices=["bolatar", "fironex"],
+                   help="which layer-list design --mixer-compare measures")
+    p.add_argument("--mixer-no-llama", action="store_true",
+                   help="--mixer-compare without the Llama runs (profiling)")
     p.add_argument("--mixer-sizes", default="small,medium",
                    help="comma list of benchmarks/mixer_compare.py SIZES")
     p.add_argument("--moe-ep", action="store_true",
@@ -461,7 +466,8 @@ def main():
         sys.path.insert(0, os.path.join(os.path.dirname(
             os.path.abspath(__file__)), "benchmarks"))
         import mixer_compare
-        mixer_compare.run(args.mixer_sizes.split(","), device)
+        mixer_compare.run(args.mixer_sizes.split(","), device,
+                          args.mixer_model, not args.mixer_no_llama)
         return
     if world > 1:
         dist.init_process_group("nccl" if device.startswith("cuda") else "gloo")

@@ -1,9 +1,10 @@
-"""Prefill and decode throughput of the layer-list (Bolatar) design beside
-the dense-attention Llama layout at equal width, depth, feed-forward size
-and vocabulary, random weights, one GPU, through the engine's own
-add_request/step loop (chunked prefill, then hipGraph decode).
+"""Prefill and decode throughput of a layer-list design (Bolatar or
+Fironex) beside the dense-attention Llama layout at equal width, depth,
+feed-forward size and vocabulary, random weights, one GPU, through the
+engine's own add_request/step loop (chunked prefill, then hipGraph decode).
 
     python bench.py --mixer-compare [--mixer-sizes small,medium]
+                    [--mixer-model bolatar|fironex]
 
 Prints one JSON line: per size and model, prefill tokens/s (B prompts of
 ISL tokens until every request has its first token) and decode tokens/s
@@ -52,6 +53,42 @@ def bolatar_config(width, layers, ff):
                        layer_specs=specs, embed_scale=1.0, logit_softcap=30.0,
                        intermediate_size=0, num_q_heads=1, num_kv_heads=1,
                        head_dim=1)
+
+
+def fironex_config(width, layers, ff):
+    """Layer pattern: differential attention under a 1024-token window,
+    latent attention, a second latent layer on the first one's cache, and
+    a gated linear recurrent unit; head sizes of current models."""
+    from dynamo_amd.engine.config import ModelConfig
+    H = width // 128
+    mlp = {"kind": "dense", "ff": ff}
+    rot = {"base": 500000.0, "dims": 64,
+           "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0,
+                       "original": 8192}}
+    specs = []
+    for i in range(layers):
+        k = i % 4
+        if k == 0:
+            specs.append({"type": "attention", "mlp": mlp, "mixer": {
+                "heads": H, "kv_heads": max(1, H // 4), "dim": 64,
+                "vdim": 128, "scale": 0.125, "diff": 0.5,
+                "mask": {"size": 1024}, "rot": rot}})
+        elif k in (1, 2):
+            m = {"heads": H, "dim": 128, "rot_dim": 64, "vdim": 128,
+                 "kv_rank": 512, "scale": 192 ** -0.5,
+                 "rot": {"base": 10000.0, "dims": 64}}
+            if k == 2:
+                m["kv_from"] = i - 1
+            specs.append({"type": "latent_attention", "mlp": mlp, "mixer": m})
+        else:
+            specs.append({"type": "rglru", "mlp": mlp, "mixer": {
+                "width": width, "blocks": H, "conv": 4}})
+    return ModelConfig(name=f"fironex-w{width}", arch="fironex",
+                       hidden_size=width, vocab_size=VOCAB, max_position=8192,
+                       num_layers=layers, rms_eps=1e-6, residual_mult=0.7,
+                       tie_embeddings=True, norm="layernorm",
+                       layer_specs=specs, intermediate_size=0, num_q_heads=1,
+                       num_kv_heads=1, head_dim=1)
 
 
 def llama_config(width, layers, ff):
@@ -123,16 +160,18 @@ def measure(mc, s, device):
     return out
 
 
-def run(sizes, device="cuda:0"):
+def run(sizes, device="cuda:0", model="bolatar", with_llama=True):
     res = {}
+    make = {"bolatar": bolatar_config, "fironex": fironex_config}[model]
     for name in sizes:
         s = SIZES[name]
         args = (s["width"], s["layers"], s["ff"])
         res[name] = {
             "shape": {k: s[k] for k in ("width", "layers", "ff", "prompts",
                                         "isl", "conc")},
-            "bolatar": measure(bolatar_config(*args), s, device),
-            "llama": measure(llama_config(*args), s, device)}
+            model: measure(make(*args), s, device)}
+        if with_llama:
+            res[name]["llama"] = measure(llama_config(*args), s, device)
         print(f"# {name}: {json.dumps(res[name])}", flush=True)
     print(json.dumps({"metric": "mixer_compare", "dtype": "bf16",
                       "data": "synthetic", "sizes": res}), flush=True)
