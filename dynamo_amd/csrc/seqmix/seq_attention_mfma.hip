@@ -1,16 +1,22 @@
-// Prompt-portion attention for the distance-biased softmax attention, on the
-// matrix cores (bf16 only): scores and the weighted sum are
-// mfma_f32_16x16x32_bf16 products, everything between them is fp32.
+// Prompt-portion softmax attention over the paged cache on the matrix cores
+// (bf16 only): scores and the weighted sum are mfma_f32_16x16x32_bf16
+// products, everything between them is fp32. Options: a logarithmic
+// distance bias with a query temperature, a sliding window, several key
+// maps per kv head, values that alias the head of the key rows (latent
+// attention), fp32 output.
 //
 // A workgroup (4 waves) owns a tile of up to 64 consecutive rows of one
-// sequence and one query head; each wave owns 16 rows. Keys and values of
-// the kv head are walked in blocks of 64: K rows are staged in LDS as they
-// lie in the page (zero padded to a multiple of 32 channels), V is staged
-// transposed (channel-major) so that the B operand of the second product
-// is a 16-byte run of keys. The fp32 scores get the row's temperature and
-// scale, the log distance penalty and the causal mask, then an online
-// softmax; the weights pass through LDS as a bf16 hi + lo pair to become
-// the A operand of two products.
+// sequence and one (query head, key map); each wave owns 16 rows. Keys and
+// values of the kv head are walked in blocks of 64 keys. Key channels are
+// staged in LDS in chunks of at most 128 channels as they lie in the page
+// (zero padded to multiples of 32), the partial scores accumulating over
+// the chunks; values are staged transposed (channel-major), again at most
+// 128 channels at a time, so that the B operand of the second product is a
+// 16-byte run of keys. Large rows (a 576-wide latent row with 512 value
+// channels) therefore need no more LDS than small ones. The fp32 scores
+// get the row's temperature and scale, the distance penalty and the mask,
+// then an online softmax; the weights pass through LDS as a bf16 hi + lo
+// pair to become the A operand of two products.
 //
 // Fragment layouts of mfma_f32_16x16x32_bf16 (lane l, lr = l % 16,
 // lg = l / 16):  A: A[row = lr][k = 8 lg + i], i = 0..7
@@ -27,40 +33,56 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 constexpr int BN = 64;    // keys per block
 constexpr int PADE = 8;   // padding elements per LDS row (16 bytes)
 
-// KC = padded key size / 32, DN = padded value size / 16
-template <int KC, int DN>
-__global__ __launch_bounds__(256) void biased_attention_mfma_kernel(
-    bf16_t* __restrict__ out,  // [T, H, dv]
-    const bf16_t* __restrict__ proj, int proj_stride, int off_q,
-    const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
-    const int* __restrict__ page_table, int table_stride,
-    const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
-    const int* __restrict__ tok_seq, const int* __restrict__ positions,
-    const float* __restrict__ r1, const float* __restrict__ r2, int H, int G,
-    int dk, int dv, int ps, float scale, float temp_coef, int temp_every,
-    int has_bias) {
-  constexpr int DKP = KC * 32, DVP = DN * 16;
-  constexpr int KS = DKP + PADE;  // k_lds row stride (elements)
-  constexpr int VS = BN + PADE;   // vt_lds / p_lds row stride
-  extern __shared__ __attribute__((aligned(16))) short smem[];
-  short* k_lds = smem;                  // [BN][KS]
-  short* vt_lds = k_lds + BN * KS;      // [DVP][VS]
-  short* p_lds = vt_lds + DVP * VS;     // [4][16][VS]
+template <typename TO> DEVINL TO out_cast(float f);
+template <> DEVINL float out_cast<float>(float f) { return f; }
+template <> DEVINL bf16_t out_cast<bf16_t>(float f) { return from_f<bf16_t>(f); }
 
-  const int tile = blockIdx.x, h = blockIdx.y;
+struct MfmaArgs {
+  const bf16_t* proj; int proj_stride; int off_q;
+  const bf16_t* kcache; const bf16_t* vcache;
+  const int* page_table; int table_stride;
+  const int* tile_row0; const int* tile_rows;
+  const int* tok_seq; const int* positions;
+  const float* r1; const float* r2;
+  int H, G, dk, dv, ps;
+  float scale, temp_coef; int temp_every, has_bias;
+  int kmaps, krow, vrow, window;
+};
+
+// KC = padded key size / 32, DN = padded value size / 16
+template <int KC, int DN, typename TO>
+__global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
+    TO* __restrict__ out,  // [T, H, kmaps, dv]
+    const MfmaArgs a) {
+  constexpr int KCH = KC < 4 ? KC : 4;       // key chunk: KCH * 32 channels
+  constexpr int NKCH = (KC + KCH - 1) / KCH;
+  constexpr int DCH = DN < 8 ? DN : 8;       // value chunk: DCH * 16 channels
+  constexpr int NDCH = (DN + DCH - 1) / DCH;
+  constexpr int KS = KCH * 32 + PADE;  // k_lds row stride (elements)
+  constexpr int VS = BN + PADE;        // vt_lds / p_lds row stride
+  static_assert(BN * KS >= 4 * 16 * VS, "the K block also holds the lo weights");
+  extern __shared__ __attribute__((aligned(16))) short smem[];
+  short* k_lds = smem;                    // [BN][KS]
+  short* vt_lds = k_lds + BN * KS;        // [DCH * 16][VS]
+  short* p_lds = vt_lds + DCH * 16 * VS;  // [4][16][VS]
+
+  const int H = a.H, G = a.G, dk = a.dk, dv = a.dv, ps = a.ps;
+  const int tile = blockIdx.x;
+  const int h = blockIdx.y / a.kmaps, map = blockIdx.y % a.kmaps;
   const int g = h / (H / G);
-  const int row0 = tile_row0[tile], nrows = tile_rows[tile];
+  const int koff = map * dk;
+  const int row0 = a.tile_row0[tile], nrows = a.tile_rows[tile];
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int lr = lane & 15, lg = lane >> 4;
-  const int* table = page_table + (int64_t)tok_seq[row0] * table_stride;
+  const int* table = a.page_table + (int64_t)a.tok_seq[row0] * a.table_stride;
 
   // ---- Q fragments of row wid*16 + lr (zero beyond dk / beyond the tile)
   bf16x8_t q_frag[KC];
   {
     const int arow = wid * 16 + lr;
     const bool ok = arow < nrows;
-    const bf16_t* q =
-        proj + (int64_t)(row0 + (ok ? arow : 0)) * proj_stride + off_q + h * dk;
+    const bf16_t* q = a.proj + (int64_t)(row0 + (ok ? arow : 0)) * a.proj_stride +
+                      a.off_q + (h * a.kmaps + map) * dk;
 #pragma unroll
     for (int kc = 0; kc < KC; kc++) {
       short8_t v;
@@ -80,15 +102,19 @@ __global__ __launch_bounds__(256) void biased_attention_mfma_kernel(
   for (int r = 0; r < 4; r++) {
     const int cr = wid * 16 + lg * 4 + r;
     ok_r[r] = cr < nrows;
-    pos_r[r] = ok_r[r] ? positions[row0 + cr] : 0;  // key 0 always exists
+    pos_r[r] = ok_r[r] ? a.positions[row0 + cr] : 0;
     float temp = 1.f;
-    if (temp_coef != 0.f)
-      temp += temp_coef * logf((float)((pos_r[r] + 1) / temp_every) + 1.f);
-    qmul[r] = temp * scale;
+    if (a.temp_coef != 0.f)
+      temp += a.temp_coef * logf((float)((pos_r[r] + 1) / a.temp_every) + 1.f);
+    qmul[r] = temp * a.scale;
   }
-  const float b1 = has_bias ? r1[h] : 0.f;
-  const float b2 = has_bias ? r2[h] : 0.f;
-  const int kv_end = positions[row0 + nrows - 1] + 1;  // rows are in order
+  const float b1 = a.has_bias ? a.r1[h] : 0.f;
+  const float b2 = a.has_bias ? a.r2[h] : 0.f;
+  const int kv_end = a.positions[row0 + nrows - 1] + 1;  // rows are in order
+  // the first key any row of the tile sees
+  const int window = a.window;
+  const int kv_begin =
+      window > 0 ? max(0, a.positions[row0] - window + 1) : 0;
 
   float m[4], l[4];
   f32x4_t acc_o[DN];
@@ -100,51 +126,42 @@ __global__ __launch_bounds__(256) void biased_attention_mfma_kernel(
 #pragma unroll
   for (int d = 0; d < DN; d++) acc_o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  const int kvecs = DKP / 8, vvecs = DVP / 8;
-  for (int t0 = 0; t0 < kv_end; t0 += BN) {
-    __syncthreads();  // the previous block's readers are done
-    // ---- stage K [BN][DKP] and V^T [DVP][BN]; zeros past dk, dv, kv_end
-    for (int slot = threadIdx.x; slot < BN * kvecs; slot += 256) {
-      const int row = slot / kvecs, v = slot - row * kvecs;
-      const int j = t0 + row;
-      short8_t x{};
-      if (j < kv_end && v * 8 < dk) {
-        const int64_t page = table[j / ps];
-        x = *reinterpret_cast<const short8_t*>(
-            kcache + ((page * G + g) * ps + (j % ps)) * dk + v * 8);
-      }
-      *reinterpret_cast<short8_t*>(k_lds + row * KS + v * 8) = x;
-    }
-    // consecutive threads take consecutive keys of one channel group, so
-    // the transposed 2-byte LDS writes fall in consecutive banks
-    for (int slot = threadIdx.x; slot < BN * vvecs; slot += 256) {
-      const int v = slot / BN, row = slot - v * BN;
-      const int j = t0 + row;
-      short8_t x{};
-      if (j < kv_end && v * 8 < dv) {
-        const int64_t page = table[j / ps];
-        x = *reinterpret_cast<const short8_t*>(
-            vcache + ((page * G + g) * ps + (j % ps)) * dv + v * 8);
-      }
-#pragma unroll
-      for (int e = 0; e < 8; e++) vt_lds[(v * 8 + e) * VS + row] = x[e];
-    }
-    __syncthreads();
-
-    // ---- S = Q K^T: block n covers keys t0 + 16 n + lr
+  for (int t0 = (kv_begin / BN) * BN; t0 < kv_end; t0 += BN) {
+    // ---- S = Q K^T over key-channel chunks: block n covers keys
+    //      t0 + 16 n + lr
     f32x4_t s[4];
 #pragma unroll
-    for (int n = 0; n < 4; n++) {
-      f32x4_t a{0.f, 0.f, 0.f, 0.f};
+    for (int n = 0; n < 4; n++) s[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kc = 0; kc < KC; kc++) {
-        const short8_t kb = *reinterpret_cast<const short8_t*>(
-            k_lds + (n * 16 + lr) * KS + kc * 32 + lg * 8);
-        short8_t tmp = kb;
-        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-            q_frag[kc], *reinterpret_cast<bf16x8_t*>(&tmp), a, 0, 0, 0);
+    for (int cc = 0; cc < NKCH; cc++) {
+      __syncthreads();  // the previous readers of k_lds are done
+      constexpr int kvecs = KCH * 4;  // 16-byte pieces per staged row
+      for (int slot = threadIdx.x; slot < BN * kvecs; slot += 256) {
+        const int row = slot / kvecs, v = slot - row * kvecs;
+        const int j = t0 + row;
+        const int ch = (cc * KCH * 4 + v) * 8;
+        short8_t x{};
+        if (j < kv_end && ch < dk) {
+          const int64_t page = table[j / ps];
+          x = *reinterpret_cast<const short8_t*>(
+              a.kcache + ((page * G + g) * ps + (j % ps)) * a.krow + koff + ch);
+        }
+        *reinterpret_cast<short8_t*>(k_lds + row * KS + v * 8) = x;
       }
-      s[n] = a;
+      __syncthreads();
+#pragma unroll
+      for (int n = 0; n < 4; n++) {
+#pragma unroll
+        for (int kc = 0; kc < KCH; kc++) {
+          if (cc * KCH + kc < KC) {
+            short8_t kb = *reinterpret_cast<const short8_t*>(
+                k_lds + (n * 16 + lr) * KS + kc * 32 + lg * 8);
+            s[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                q_frag[cc * KCH + kc], *reinterpret_cast<bf16x8_t*>(&kb), s[n],
+                0, 0, 0);
+          }
+        }
+      }
     }
     // ---- fp32: scale, penalty, mask, online softmax (rows 4 lg + r)
     float p[4][4];
@@ -155,8 +172,9 @@ __global__ __launch_bounds__(256) void biased_attention_mfma_kernel(
       for (int n = 0; n < 4; n++) {
         const int j = t0 + n * 16 + lr;
         float x = s[n][r] * qmul[r];
-        if (has_bias) x -= b1 * log1pf(b2 * (float)max(pos_r[r] - j, 0));
-        x = j <= pos_r[r] ? x : -INFINITY;
+        if (a.has_bias) x -= b1 * log1pf(b2 * (float)max(pos_r[r] - j, 0));
+        const bool seen = j <= pos_r[r] && (window == 0 || j > pos_r[r] - window);
+        x = seen ? x : -INFINITY;
         p[n][r] = x;
         mt = fmaxf(mt, x);
       }
@@ -164,12 +182,15 @@ __global__ __launch_bounds__(256) void biased_attention_mfma_kernel(
       mt = fmaxf(mt, __shfl_xor(mt, 2, 64));
       mt = fmaxf(mt, __shfl_xor(mt, 4, 64));
       mt = fmaxf(mt, __shfl_xor(mt, 8, 64));
-      const float mn = fmaxf(m[r], mt);  // finite from the first block on
-      const float corr = expf(m[r] - mn);
+      // a row may see nothing of the first blocks (window): then every
+      // weight is 0 and the running maximum stays -inf
+      const float mn = fmaxf(m[r], mt);
+      const float base = mn == -INFINITY ? 0.f : mn;
+      const float corr = expf(m[r] - base);
       float rs = 0.f;
 #pragma unroll
       for (int n = 0; n < 4; n++) {
-        p[n][r] = expf(p[n][r] - mn);
+        p[n][r] = expf(p[n][r] - base);
         rs += p[n][r];
       }
       rs += __shfl_xor(rs, 1, 64);
@@ -197,24 +218,46 @@ __global__ __launch_bounds__(256) void biased_attention_mfma_kernel(
         pw[(lg * 4 + r) * VS + n * 16 + lr] = (short)hi;
         pl[(lg * 4 + r) * VS + n * 16 + lr] = (short)lo;
       }
-    __syncthreads();
-    // ---- O += P V
+    // ---- O += P V over value-channel chunks, V staged transposed
 #pragma unroll
-    for (int kt = 0; kt < 2; kt++) {
-      short8_t pa = *reinterpret_cast<const short8_t*>(
-          pw + lr * VS + kt * 32 + lg * 8);
-      short8_t pb = *reinterpret_cast<const short8_t*>(
-          pl + lr * VS + kt * 32 + lg * 8);
+    for (int vc = 0; vc < NDCH; vc++) {
+      if (vc) __syncthreads();  // the previous chunk's readers are done
+      // consecutive threads take consecutive keys of one channel group, so
+      // the transposed 2-byte LDS writes fall in consecutive banks
+      constexpr int vvecs = DCH * 2;
+      for (int slot = threadIdx.x; slot < BN * vvecs; slot += 256) {
+        const int v = slot / BN, row = slot - v * BN;
+        const int j = t0 + row;
+        const int ch = (vc * DCH * 2 + v) * 8;
+        short8_t x{};
+        if (j < kv_end && ch < dv) {
+          const int64_t page = table[j / ps];
+          x = *reinterpret_cast<const short8_t*>(
+              a.vcache + ((page * G + g) * ps + (j % ps)) * a.vrow + ch);
+        }
 #pragma unroll
-      for (int d = 0; d < DN; d++) {
-        short8_t vb = *reinterpret_cast<const short8_t*>(
-            vt_lds + (d * 16 + lr) * VS + kt * 32 + lg * 8);
-        acc_o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-            *reinterpret_cast<bf16x8_t*>(&pa),
-            *reinterpret_cast<bf16x8_t*>(&vb), acc_o[d], 0, 0, 0);
-        acc_o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-            *reinterpret_cast<bf16x8_t*>(&pb),
-            *reinterpret_cast<bf16x8_t*>(&vb), acc_o[d], 0, 0, 0);
+        for (int e = 0; e < 8; e++) vt_lds[(v * 8 + e) * VS + row] = x[e];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++) {
+        short8_t pa = *reinterpret_cast<const short8_t*>(
+            pw + lr * VS + kt * 32 + lg * 8);
+        short8_t pb = *reinterpret_cast<const short8_t*>(
+            pl + lr * VS + kt * 32 + lg * 8);
+#pragma unroll
+        for (int d = 0; d < DCH; d++) {
+          if (vc * DCH + d < DN) {
+            short8_t vb = *reinterpret_cast<const short8_t*>(
+                vt_lds + (d * 16 + lr) * VS + kt * 32 + lg * 8);
+            acc_o[vc * DCH + d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                *reinterpret_cast<bf16x8_t*>(&pa),
+                *reinterpret_cast<bf16x8_t*>(&vb), acc_o[vc * DCH + d], 0, 0, 0);
+            acc_o[vc * DCH + d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                *reinterpret_cast<bf16x8_t*>(&pb),
+                *reinterpret_cast<bf16x8_t*>(&vb), acc_o[vc * DCH + d], 0, 0, 0);
+          }
+        }
       }
     }
   }
@@ -223,69 +266,124 @@ __global__ __launch_bounds__(256) void biased_attention_mfma_kernel(
   for (int r = 0; r < 4; r++) {
     if (!ok_r[r]) continue;
     const float inv = 1.f / l[r];
-    bf16_t* o = out + ((int64_t)(row0 + wid * 16 + lg * 4 + r) * H + h) * dv;
+    TO* o = out + (((int64_t)(row0 + wid * 16 + lg * 4 + r) * H + h) * a.kmaps +
+                   map) * dv;
 #pragma unroll
     for (int d = 0; d < DN; d++) {
       const int ch = d * 16 + lr;
-      if (ch < dv) o[ch] = from_f<bf16_t>(acc_o[d][r] * inv);
+      if (ch < dv) o[ch] = out_cast<TO>(acc_o[d][r] * inv);
     }
   }
 }
 
-template <int KC, int DN>
-void launch(dim3 grid, size_t lds, bf16_t* out, const bf16_t* proj,
-            int proj_stride, int off_q, const bf16_t* kc, const bf16_t* vc,
-            const int* pt, int pts, const int* tr0, const int* trn,
-            const int* tok_seq, const int* positions, const float* r1,
-            const float* r2, int H, int G, int dk, int dv, int ps, float scale,
-            float temp_coef, int temp_every, int has_bias) {
-  hipLaunchKernelGGL((biased_attention_mfma_kernel<KC, DN>), grid, dim3(256),
-                     lds, cur_stream(), out, proj, proj_stride, off_q, kc, vc,
-                     pt, pts, tr0, trn, tok_seq, positions, r1, r2, H, G, dk,
-                     dv, ps, scale, temp_coef, temp_every, has_bias);
+inline size_t lds_bytes(int KC, int DN) {
+  const int KCH = KC < 4 ? KC : 4, DCH = DN < 8 ? DN : 8;
+  return (size_t)(BN * (KCH * 32 + PADE) + DCH * 16 * (BN + PADE) +
+                  4 * 16 * (BN + PADE)) * sizeof(short);
 }
 
-inline size_t lds_bytes(int KC, int DN) {
-  return (size_t)(BN * (KC * 32 + PADE) + DN * 16 * (BN + PADE) +
-                  4 * 16 * (BN + PADE)) * sizeof(short);
+template <int KC, int DN, typename TO>
+void launch(dim3 grid, TO* out, const MfmaArgs& a) {
+  hipLaunchKernelGGL((paged_attention_mfma_kernel<KC, DN, TO>), grid, dim3(256),
+                     lds_bytes(KC, DN), cur_stream(), out, a);
+}
+
+// padded sizes the kernel is built for: key chunks of 32, value chunks of 16
+inline int pick_kc(int dk) {
+  for (int kc : {2, 4, 6, 8, 10, 18})
+    if (dk <= kc * 32) return kc;
+  return 0;
+}
+inline int pick_dn(int dv) {
+  for (int dn : {4, 8, 16, 32})
+    if (dv <= dn * 16) return dn;
+  return 0;
+}
+
+template <typename TO>
+bool dispatch(int KC, int DN, dim3 grid, TO* out, const MfmaArgs& a) {
+#define CASE(KC_, DN_)                                  \
+  if (KC == KC_ && DN == DN_) {                         \
+    launch<KC_, DN_, TO>(grid, out, a);                 \
+    return true;                                        \
+  }
+  CASE(2, 4) CASE(2, 8) CASE(2, 16)
+  CASE(4, 4) CASE(4, 8) CASE(4, 16)
+  CASE(8, 4) CASE(8, 8) CASE(8, 16)
+  if constexpr (std::is_same<TO, float>::value) {
+    CASE(6, 8) CASE(10, 16) CASE(18, 32)
+  }
+#undef CASE
+  return false;
+}
+
+inline bool combo_ok(int KC, int DN, bool f32out) {
+  if (KC == 0 || DN == 0) return false;
+  if (KC <= 8 && KC != 6 && DN <= 16) return true;
+  return f32out && ((KC == 6 && DN == 8) || (KC == 10 && DN == 16) ||
+                    (KC == 18 && DN == 32));
 }
 
 }  // namespace
 
 // Whether the matrix-core kernel covers these sizes (bf16 caches only).
+bool paged_attention_mfma_supported(int64_t dk, int64_t dv, bool f32out) {
+  if (dk % 8 || dv % 8 || dk < 8 || dv < 8) return false;
+  return combo_ok(pick_kc((int)dk), pick_dn((int)dv), f32out);
+}
 bool biased_attention_mfma_supported(int64_t dk, int64_t dv) {
-  if (dk % 8 || dv % 8 || dk > 256 || dv > 256) return false;
-  const int KC = dk <= 64 ? 2 : (dk <= 128 ? 4 : 8);
-  const int DN = dv <= 64 ? 4 : (dv <= 128 ? 8 : 16);
-  return lds_bytes(KC, DN) <= 64 * 1024;
+  return paged_attention_mfma_supported(dk, dv, false);
 }
 
 // Rows are given as tiles: tile i covers rows [tile_row0[i], + tile_rows[i])
-// (at most 64, consecutive positions of one sequence).
-void biased_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
-                           torch::Tensor kcache, torch::Tensor vcache,
-                           torch::Tensor page_table, torch::Tensor tile_row0,
-                           torch::Tensor tile_rows, int64_t max_tile_rows,
-                           torch::Tensor tok_seq, torch::Tensor positions,
-                           c10::optional<torch::Tensor> r1,
-                           c10::optional<torch::Tensor> r2, double scale,
-                           double temp_coef, int64_t temp_every) {
-  const int T_ = out.size(0), H = out.size(1), dv = out.size(2);
-  const int G = kcache.size(1), ps = kcache.size(2), dk = kcache.size(3);
+// (at most 64, consecutive positions of one sequence). out [T, H, kmaps, dv]
+// fp32 or bf16; values from vcache, or from the head of the key rows.
+void paged_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
+                          torch::Tensor kcache,
+                          c10::optional<torch::Tensor> vcache,
+                          torch::Tensor page_table, torch::Tensor tile_row0,
+                          torch::Tensor tile_rows, int64_t max_tile_rows,
+                          torch::Tensor tok_seq, torch::Tensor positions,
+                          c10::optional<torch::Tensor> r1,
+                          c10::optional<torch::Tensor> r2, double scale,
+                          double temp_coef, int64_t temp_every, int64_t kmaps,
+                          int64_t window) {
+  SEQ_CHECK(out.dim() == 4 && out.is_contiguous() && out.size(2) == kmaps,
+            "mfma attention out [T, H, maps, dv]");
+  const int T_ = out.size(0), H = out.size(1), dv = out.size(3);
+  const int G = kcache.size(1), ps = kcache.size(2), krow = kcache.size(3);
+  SEQ_CHECK(kmaps >= 1 && krow % kmaps == 0 && window >= 0, "key maps/window");
+  const int dk = krow / kmaps;
   const int NT = tile_row0.size(0);
-  SEQ_CHECK(out.scalar_type() == torch::kBFloat16 && out.is_contiguous() &&
+  const bool f32out = out.scalar_type() == torch::kFloat;
+  SEQ_CHECK((f32out || out.scalar_type() == torch::kBFloat16) &&
                 proj.scalar_type() == torch::kBFloat16 &&
-                kcache.scalar_type() == torch::kBFloat16 &&
-                vcache.scalar_type() == torch::kBFloat16, "mfma attention is bf16");
-  SEQ_CHECK(kcache.is_contiguous() && vcache.is_contiguous() &&
-                vcache.size(3) == dv && vcache.size(1) == G &&
-                vcache.size(2) == ps && H % G == 0, "mfma attention cache");
-  SEQ_CHECK(biased_attention_mfma_supported(dk, dv), "mfma attention sizes");
+                kcache.scalar_type() == torch::kBFloat16,
+            "mfma attention is bf16");
+  SEQ_CHECK(kcache.is_contiguous() && G >= 1 && H % G == 0,
+            "mfma attention cache");
+  const bf16_t* vptr;
+  int vrow;
+  if (vcache) {
+    SEQ_CHECK(vcache->scalar_type() == torch::kBFloat16 &&
+                  vcache->is_contiguous() && vcache->size(3) == dv &&
+                  vcache->size(1) == G && vcache->size(2) == ps &&
+                  vcache->size(0) == kcache.size(0), "mfma value cache");
+    vptr = cptr<bf16_t>(*vcache);
+    vrow = dv;
+  } else {
+    SEQ_CHECK(dv <= krow, "values inside the key rows");
+    vptr = cptr<bf16_t>(kcache);
+    vrow = krow;
+  }
+  SEQ_CHECK(paged_attention_mfma_supported(dk, dv, f32out),
+            "mfma attention sizes");
   SEQ_CHECK(reinterpret_cast<uintptr_t>(kcache.data_ptr()) % 16 == 0 &&
-                reinterpret_cast<uintptr_t>(vcache.data_ptr()) % 16 == 0,
-            "mfma attention cache alignment");
-  SEQ_CHECK(proj.stride(1) == 1 && proj.size(0) == T_ &&
-                off_q + H * dk <= proj.size(1), "mfma attention q");
+                reinterpret_cast<uintptr_t>(vptr) % 16 == 0 && krow % 8 == 0 &&
+                vrow % 8 == 0, "mfma attention cache alignment");
+  SEQ_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(0) == T_ &&
+                off_q >= 0 && off_q + H * kmaps * dk <= proj.size(1),
+            "mfma attention q");
   SEQ_CHECK(page_table.scalar_type() == torch::kInt && page_table.dim() == 2 &&
                 page_table.stride(1) == 1, "page table");
   for (const torch::Tensor* t : {&tok_seq, &positions})
@@ -297,30 +395,42 @@ void biased_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
   SEQ_CHECK(max_tile_rows >= 1 && max_tile_rows <= 64, "tile height");
   SEQ_CHECK(r1.has_value() == r2.has_value(), "bias parameters");
   if (r1)
-    SEQ_CHECK(r1->scalar_type() == torch::kFloat && r1->numel() == H &&
-                  r2->scalar_type() == torch::kFloat && r2->numel() == H,
-              "bias parameters");
+    SEQ_CHECK(kmaps == 1 && r1->scalar_type() == torch::kFloat &&
+                  r1->numel() == H && r2->scalar_type() == torch::kFloat &&
+                  r2->numel() == H, "bias parameters");
   SEQ_CHECK(temp_every >= 1, "temperature period");
   if (NT == 0) return;
-  const int KC = dk <= 64 ? 2 : (dk <= 128 ? 4 : 8);
-  const int DN = dv <= 64 ? 4 : (dv <= 128 ? 8 : 16);
-  const size_t lds = lds_bytes(KC, DN);
-#define ARGS                                                                  \
-  dim3(NT, H), lds, ptr<bf16_t>(out), cptr<bf16_t>(proj),                     \
-      (int)proj.stride(0), (int)off_q, cptr<bf16_t>(kcache),                  \
-      cptr<bf16_t>(vcache), cptr<int>(page_table), (int)page_table.stride(0), \
-      cptr<int>(tile_row0), cptr<int>(tile_rows), cptr<int>(tok_seq),         \
-      cptr<int>(positions), r1 ? cptr<float>(*r1) : nullptr,                  \
-      r2 ? cptr<float>(*r2) : nullptr, H, G, dk, dv, ps, (float)scale,        \
-      (float)temp_coef, (int)temp_every, r1 ? 1 : 0
-  if (KC == 2 && DN == 4) launch<2, 4>(ARGS);
-  else if (KC == 2 && DN == 8) launch<2, 8>(ARGS);
-  else if (KC == 2 && DN == 16) launch<2, 16>(ARGS);
-  else if (KC == 4 && DN == 4) launch<4, 4>(ARGS);
-  else if (KC == 4 && DN == 8) launch<4, 8>(ARGS);
-  else if (KC == 4 && DN == 16) launch<4, 16>(ARGS);
-  else if (KC == 8 && DN == 4) launch<8, 4>(ARGS);
-  else if (KC == 8 && DN == 8) launch<8, 8>(ARGS);
-  else TORCH_CHECK(false, "seqmix: mfma attention sizes");
-#undef ARGS
+  MfmaArgs a;
+  a.proj = cptr<bf16_t>(proj); a.proj_stride = (int)proj.stride(0);
+  a.off_q = (int)off_q;
+  a.kcache = cptr<bf16_t>(kcache); a.vcache = vptr;
+  a.page_table = cptr<int>(page_table);
+  a.table_stride = (int)page_table.stride(0);
+  a.tile_row0 = cptr<int>(tile_row0); a.tile_rows = cptr<int>(tile_rows);
+  a.tok_seq = cptr<int>(tok_seq); a.positions = cptr<int>(positions);
+  a.r1 = r1 ? cptr<float>(*r1) : nullptr;
+  a.r2 = r2 ? cptr<float>(*r2) : nullptr;
+  a.H = H; a.G = G; a.dk = dk; a.dv = dv; a.ps = ps;
+  a.scale = (float)scale; a.temp_coef = (float)temp_coef;
+  a.temp_every = (int)temp_every; a.has_bias = r1 ? 1 : 0;
+  a.kmaps = (int)kmaps; a.krow = krow; a.vrow = vrow; a.window = (int)window;
+  const int KC = pick_kc(dk), DN = pick_dn(dv);
+  const dim3 grid(NT, H * kmaps);
+  const bool ok = f32out ? dispatch<float>(KC, DN, grid, ptr<float>(out), a)
+                         : dispatch<bf16_t>(KC, DN, grid, ptr<bf16_t>(out), a);
+  TORCH_CHECK(ok, "seqmix: mfma attention sizes");
+}
+
+void biased_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
+                           torch::Tensor kcache, torch::Tensor vcache,
+                           torch::Tensor page_table, torch::Tensor tile_row0,
+                           torch::Tensor tile_rows, int64_t max_tile_rows,
+                           torch::Tensor tok_seq, torch::Tensor positions,
+                           c10::optional<torch::Tensor> r1,
+                           c10::optional<torch::Tensor> r2, double scale,
+                           double temp_coef, int64_t temp_every) {
+  SEQ_CHECK(out.dim() == 3 && out.is_contiguous(), "mfma attention out");
+  paged_attention_mfma(out.unsqueeze(2), proj, off_q, kcache, vcache,
+                       page_table, tile_row0, tile_rows, max_tile_rows, tok_seq,
+                       positions, r1, r2, scale, temp_coef, temp_every, 1, 0);
 }

@@ -68,6 +68,13 @@ void rglru_scan(Tensor out, Tensor u, Tensor gates, Tensor br, Tensor bi,
                 Tensor lam, Tensor y, Tensor state, Tensor seq_start,
                 Tensor seq_len, Tensor seq_slot, Tensor seq_pos0, double decay);
 bool biased_attention_mfma_supported(int64_t dk, int64_t dv);
+bool paged_attention_mfma_supported(int64_t dk, int64_t dv, bool f32out);
+void paged_attention_mfma(Tensor out, Tensor proj, int64_t off_q, Tensor kcache,
+                          OptTensor vcache, Tensor page_table, Tensor tile_row0,
+                          Tensor tile_rows, int64_t max_tile_rows,
+                          Tensor tok_seq, Tensor positions, OptTensor r1,
+                          OptTensor r2, double scale, double temp_coef,
+                          int64_t temp_every, int64_t kmaps, int64_t window);
 void biased_attention_mfma(Tensor out, Tensor proj, int64_t off_q,
                            Tensor kcache, Tensor vcache, Tensor page_table,
                            Tensor tile_row0, Tensor tile_rows,
@@ -101,4 +108,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("rglru_scan", &rglru_scan);
   m.def("biased_attention_mfma_supported", &biased_attention_mfma_supported);
   m.def("biased_attention_mfma", &biased_attention_mfma);
+  m.def("paged_attention_mfma_supported", &paged_attention_mfma_supported);
+  m.def("paged_attention_mfma", &paged_attention_mfma);
 }

@@ -300,10 +300,25 @@ def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
         T = q.shape[0]
         out = torch.empty(T, H, kmaps, dv, dtype=torch.float32,
                           device=q.device)
-        hip_seq().paged_attention_rows(
-            out, q, off_q, kcache, vcache, sb.page_table, sb.tok_seq,
-            positions, sb.seq_len, None, None, float(scale), 0.0, 1,
-            int(kmaps), int(window))
+        m = hip_seq()
+        # prompt portions in bf16 go to the MFMA kernel when the row sizes
+        # fit it; decoded tokens, fp32 and other sizes take the row kernel
+        krow = kcache.shape[3]
+        tiled = (sb.tiles is not None and q.dtype == torch.bfloat16
+                 and m.paged_attention_mfma_supported(krow // kmaps, dv, True)
+                 and krow % 8 == 0 and kcache.data_ptr() % 16 == 0
+                 and (vcache is None or vcache.data_ptr() % 16 == 0))
+        nrow = sb.num_decode if tiled else T
+        if nrow:
+            m.paged_attention_rows(
+                out[:nrow], q[:nrow], off_q, kcache, vcache, sb.page_table,
+                sb.tok_seq[:nrow], positions[:nrow], sb.seq_len, None, None,
+                float(scale), 0.0, 1, int(kmaps), int(window))
+        if tiled and sb.tiles[0].numel():
+            m.paged_attention_mfma(
+                out, q, off_q, kcache, vcache, sb.page_table, sb.tiles[0],
+                sb.tiles[1], 64, sb.tok_seq, positions, None, None,
+                float(scale), 0.0, 1, int(kmaps), int(window))
         return out
     return seq_ref.paged_attention_rows(q, off_q, H, kmaps, kcache, vcache,
                                         dv, positions, sb, scale, window)

@@ -223,7 +223,7 @@ def test_sharp_latent_attention_really_looks_far():
     assert far > 0.2
 
 
-def _window_case(W_size, i, j, dk=8, dv=6, ps=4, strong=40.0, seed=0):
+def _window_case(W_size, i, j, dk=8, dv=6, ps=4, strong=40.0, seed=0):  # noqa
     """One kv head, two maps, T = i + 1 tokens. Map 0's key j points along
     query i with a large norm, so it takes all the weight if visible; map 1
     likewise for key j + 1. Returns q, k, v as [T, ...] tensors."""
@@ -434,6 +434,139 @@ def test_unused_checkpoint_tensor_is_an_error(tmp_path):
     path = U.write_checkpoint(tmp_path, cfg, W)
     with pytest.raises(ValueError):
         U.make_engine(path, "cpu")
+
+
+# -- bf16 prompt portions on the matrix cores ---------------------------------
+def _paged(k, v, ps, extra=3, seed=0):
+    """Scatter [T, G, d] keys (and values) over pages in a random order."""
+    T, G = k.shape[0], k.shape[1]
+    npg = -(-T // ps)
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(npg + extra, generator=g)[:npg]
+    kc = torch.zeros(npg + extra, G, ps, k.shape[2], dtype=k.dtype)
+    vc = None if v is None else torch.zeros(npg + extra, G, ps, v.shape[2],
+                                            dtype=v.dtype)
+    for t in range(T):
+        kc[perm[t // ps], :, t % ps] = k[t]
+        if v is not None:
+            vc[perm[t // ps], :, t % ps] = v[t]
+    return kc, vc, perm.to(torch.int32)
+
+
+def _prompt_batch(spans, tables, dev, tiled):
+    """SeqBatch of prompt portions [(rows, first position)], one per page
+    table row, with or without 64-row tiles."""
+    from dynamo_amd.ops import seq as sops
+    tok_seq, start, host, t0, tn = [], 0, [], [], []
+    for si, (n, pos0) in enumerate(spans):
+        host.append((start, n, si, pos0))
+        tok_seq += [si] * n
+        for q0 in range(0, n, 64):
+            t0.append(start + q0)
+            tn.append(min(64, n - q0))
+        start += n
+    maxp = max(len(t) for t in tables)
+    pt = torch.zeros(len(tables), maxp, dtype=torch.int32)
+    for i, t in enumerate(tables):
+        pt[i, :len(t)] = t
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)  # noqa: E731
+    cols = list(zip(*host))
+    pos = torch.cat([torch.arange(p0, p0 + n) for n, p0 in spans]).to(
+        torch.int32).to(dev)
+    sb = sops.SeqBatch(i32(tok_seq), i32(cols[0]), i32(cols[1]), i32(cols[2]),
+                       i32(cols[3]), page_table=pt.to(dev), num_decode=0,
+                       tiles=(i32(t0), i32(tn)) if tiled else None)
+    return sb, pos
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,dk,dv,kmaps,window,alias", [
+    (4, 2, 64, 128, 2, 100, False),     # differential heads under a window
+    (6, 3, 24, 40, 2, 19, False),       # sizes padded inside the kernel
+    (2, 1, 128, 64, 1, 0, False),       # plain grouped attention
+    (3, 1, 192, 128, 1, 0, True),       # latent rows: values alias keys
+    (2, 1, 320, 256, 1, 0, True),
+    (4, 1, 576, 512, 1, 0, True),
+    (2, 2, 16, 8, 2, 1, False),         # a window of one token
+])
+def test_mfma_prompt_attention_matches_row_kernel(H, G, dk, dv, kmaps, window,
+                                                  alias):
+    """bf16 prompt portions (two sequences, one continued from position 70
+    so that tiles start inside a page and inside the window) through the
+    matrix-core kernel against the fp32-accumulating row kernel and the
+    oracle."""
+    from dynamo_amd.ops import seq as sops
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(dk + dv)
+    ps = 16
+    lens = [(130, 0), (75, 70)]          # (rows this step, first position)
+    krow = kmaps * dk
+    ks, vs, tabs, qs = [], [], [], []
+    for n, p0 in lens:
+        T = n + p0
+        k = (torch.randn(T, G, krow, generator=g) * 0.7).to(torch.bfloat16)
+        v = None if alias else torch.randn(T, G, dv, generator=g).to(torch.bfloat16)
+        ks.append(k)
+        vs.append(v)
+        qs.append((torch.randn(n, H * krow, generator=g) * 0.7).to(torch.bfloat16))
+    # one cache for both sequences: pages of the second follow the first's
+    kc0, vc0, t0 = _paged(ks[0], vs[0], ps, seed=1)
+    kc1, vc1, t1 = _paged(ks[1], vs[1], ps, seed=2)
+    kc = torch.cat([kc0, kc1])
+    vc = None if alias else torch.cat([vc0, vc1])
+    tabs = [t0, t1 + kc0.shape[0]]
+    q = torch.cat(qs)
+    outs = []
+    for tiled in (False, True):
+        sb, pos = _prompt_batch(lens, tabs, dev, tiled)
+        outs.append(sops.paged_attention_rows(
+            q.to(dev), 0, H, kmaps, kc.to(dev), None if alias else vc.to(dev),
+            dv, pos, sb, 0.11, window).cpu())
+    assert torch.isfinite(outs[1]).all()
+    scale = float(outs[0].abs().max())
+    assert float((outs[0] - outs[1]).abs().max()) < 2e-3 * scale
+    # the oracle on the same bf16 inputs, last rows of each sequence
+    row = 0
+    for (n, p0), k, v, qq in zip(lens, ks, vs, qs):
+        T = n + p0
+        kd = k.double().view(T, G, kmaps, dk)
+        vd = kd.reshape(T, G, krow)[:, :, :dv] if alias else v.double()
+        for h in (0, H - 1):
+            for mp in range(kmaps):
+                qfull = torch.zeros(T, dk, dtype=torch.float64)
+                qfull[p0:] = qq.double().view(n, H, kmaps, dk)[:, h, mp]
+                want = oracle.masked_softmax_attention(
+                    qfull, kd[:, h // (H // G), mp], vd[:, h // (H // G)],
+                    0.11, window or None)[p0:]
+                got = outs[1][row:row + n, h, mp].double()
+                assert float((got - want).abs().max()) < 2e-3 * scale, (h, mp)
+        row += n
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("window", [5, 64, 70])
+def test_window_edges_on_the_matrix_cores(window):
+    """The dominating key just outside / just inside the window, bf16
+    prompt tiles: the last row of the last tile decides."""
+    from dynamo_amd.ops import seq as sops
+    dev = torch.device("cuda:0")
+    i = 2 * window + 37
+    for j in (i - window, i - window + 1):
+        q, k, v = _window_case(window, i, j, dk=16, dv=8, seed=window + j)
+        q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+        T = i + 1
+        kc, vc, tab = _paged(k.reshape(T, 1, -1), v, 16, seed=3)
+        sb, pos = _prompt_batch([(T, 0)], [tab], dev, True)
+        got = sops.paged_attention_rows(
+            q.reshape(T, -1).to(dev), 0, 1, 2, kc.to(dev), vc.to(dev), 8, pos,
+            sb, 0.5, window).cpu()
+        inside = j > i - window
+        hit = torch.allclose(got[-1, 0, 0], v[j, 0].float(), atol=2e-2)
+        assert hit == inside
+        want = oracle.masked_softmax_attention(
+            q[:, 0, 1].double(), k[:, 0, 1].double(), v[:, 0].double(), 0.5,
+            window)
+        assert torch.allclose(got[:, 0, 1].double(), want, atol=2e-2)
 
 
 # -- bf16 and graphs ---------------------------------------------------------
