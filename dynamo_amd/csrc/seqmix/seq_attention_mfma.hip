@@ -18,6 +18,13 @@
 // then an online softmax; the weights pass through LDS as a bf16 hi + lo
 // pair to become the A operand of two products.
 //
+// Decoded tokens use the same kernel with the roles of the tile's rows
+// changed (HEADS): a tile is one token, its rows are the query heads that
+// share a kv head (all 16, 64, 128 heads of a latent layer share the one
+// cached row, so the products are as dense as in a prompt). The keys of a
+// token are split over several workgroups; each leaves an unnormalised
+// partial result (max, sum, accumulator) that a merge kernel combines.
+//
 // Fragment layouts of mfma_f32_16x16x32_bf16 (lane l, lr = l % 16,
 // lg = l / 16):  A: A[row = lr][k = 8 lg + i], i = 0..7
 //                B: B[k = 8 lg + i][col = lr]
@@ -47,10 +54,12 @@ struct MfmaArgs {
   int H, G, dk, dv, ps;
   float scale, temp_coef; int temp_every, has_bias;
   int kmaps, krow, vrow, window;
+  // HEADS mode: rows of a tile are heads of one decoded token
+  const int* seq_len; int nsplit; float* partial;
 };
 
 // KC = padded key size / 32, DN = padded value size / 16
-template <int KC, int DN, typename TO>
+template <int KC, int DN, typename TO, bool HEADS>
 __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     TO* __restrict__ out,  // [T, H, kmaps, dv]
     const MfmaArgs a) {
@@ -68,21 +77,35 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 
   const int H = a.H, G = a.G, dk = a.dk, dv = a.dv, ps = a.ps;
   const int tile = blockIdx.x;
-  const int h = blockIdx.y / a.kmaps, map = blockIdx.y % a.kmaps;
-  const int g = h / (H / G);
+  const int gsz = H / G;
+  // prompt tiles: blockIdx.y = head * kmaps + map, rows are tokens.
+  // HEADS: blockIdx.y = ((kv head * kmaps) + map) * nhb + head block,
+  // blockIdx.x is the token and rows are the heads h0 + row.
+  const int nhb = (gsz + 63) / 64;
+  const int map = HEADS ? (blockIdx.y / nhb) % a.kmaps : blockIdx.y % a.kmaps;
+  const int g = HEADS ? blockIdx.y / (nhb * a.kmaps)
+                      : (blockIdx.y / a.kmaps) / gsz;
+  const int h = HEADS ? g * gsz + (blockIdx.y % nhb) * 64 : blockIdx.y / a.kmaps;
   const int koff = map * dk;
-  const int row0 = a.tile_row0[tile], nrows = a.tile_rows[tile];
+  const int row0 = HEADS ? tile : a.tile_row0[tile];
+  const int nrows = HEADS ? min(64, g * gsz + gsz - h) : a.tile_rows[tile];
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int lr = lane & 15, lg = lane >> 4;
-  const int* table = a.page_table + (int64_t)a.tok_seq[row0] * a.table_stride;
+  const int seq = a.tok_seq[row0];
+  if (HEADS && a.seq_len[seq] == 0) return;  // padding row (uniform exit)
+  const int* table = a.page_table + (int64_t)seq * a.table_stride;
+  const bool active = wid * 16 < nrows;  // this wave has rows (wave-uniform)
 
   // ---- Q fragments of row wid*16 + lr (zero beyond dk / beyond the tile)
   bf16x8_t q_frag[KC];
   {
     const int arow = wid * 16 + lr;
     const bool ok = arow < nrows;
-    const bf16_t* q = a.proj + (int64_t)(row0 + (ok ? arow : 0)) * a.proj_stride +
-                      a.off_q + (h * a.kmaps + map) * dk;
+    const bf16_t* q =
+        HEADS ? a.proj + (int64_t)row0 * a.proj_stride + a.off_q +
+                    ((h + (ok ? arow : 0)) * a.kmaps + map) * dk
+              : a.proj + (int64_t)(row0 + (ok ? arow : 0)) * a.proj_stride +
+                    a.off_q + (h * a.kmaps + map) * dk;
 #pragma unroll
     for (int kc = 0; kc < KC; kc++) {
       short8_t v;
@@ -102,7 +125,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   for (int r = 0; r < 4; r++) {
     const int cr = wid * 16 + lg * 4 + r;
     ok_r[r] = cr < nrows;
-    pos_r[r] = ok_r[r] ? a.positions[row0 + cr] : 0;
+    pos_r[r] = HEADS ? a.positions[row0]
+                     : (ok_r[r] ? a.positions[row0 + cr] : 0);
     float temp = 1.f;
     if (a.temp_coef != 0.f)
       temp += a.temp_coef * logf((float)((pos_r[r] + 1) / a.temp_every) + 1.f);
@@ -110,7 +134,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   }
   const float b1 = a.has_bias ? a.r1[h] : 0.f;
   const float b2 = a.has_bias ? a.r2[h] : 0.f;
-  const int kv_end = a.positions[row0 + nrows - 1] + 1;  // rows are in order
+  // prompt rows are in order; the heads of a token share its position
+  const int kv_end = a.positions[HEADS ? row0 : row0 + nrows - 1] + 1;
   // the first key any row of the tile sees
   const int window = a.window;
   const int kv_begin =
@@ -126,7 +151,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 #pragma unroll
   for (int d = 0; d < DN; d++) acc_o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  for (int t0 = (kv_begin / BN) * BN; t0 < kv_end; t0 += BN) {
+  const int kstep = HEADS ? a.nsplit : 1;
+  for (int t0 = (kv_begin / BN + (HEADS ? (int)blockIdx.z : 0)) * BN;
+       t0 < kv_end; t0 += kstep * BN) {
     // ---- S = Q K^T over key-channel chunks: block n covers keys
     //      t0 + 16 n + lr
     f32x4_t s[4];
@@ -149,6 +176,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
         *reinterpret_cast<short8_t*>(k_lds + row * KS + v * 8) = x;
       }
       __syncthreads();
+      if (active)
 #pragma unroll
       for (int n = 0; n < 4; n++) {
 #pragma unroll
@@ -239,6 +267,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
         for (int e = 0; e < 8; e++) vt_lds[(v * 8 + e) * VS + row] = x[e];
       }
       __syncthreads();
+      if (active)
 #pragma unroll
       for (int kt = 0; kt < 2; kt++) {
         short8_t pa = *reinterpret_cast<const short8_t*>(
@@ -261,6 +290,28 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       }
     }
   }
+  if (HEADS) {
+    // ---- partial result of this key split: [token, head, map, split] x
+    //      (max, sum, dv unnormalised channels)
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      if (!ok_r[r]) continue;
+      const int hh = h + wid * 16 + lg * 4 + r;
+      float* o = a.partial +
+                 ((((int64_t)row0 * H + hh) * a.kmaps + map) * a.nsplit +
+                  blockIdx.z) * (dv + 2);
+      if (lr == 0) {
+        o[0] = m[r];
+        o[1] = l[r];
+      }
+#pragma unroll
+      for (int d = 0; d < DN; d++) {
+        const int ch = d * 16 + lr;
+        if (ch < dv) o[2 + ch] = acc_o[d][r];
+      }
+    }
+    return;
+  }
   // ---- normalise and store rows 4 lg + r, channels 16 d + lr
 #pragma unroll
   for (int r = 0; r < 4; r++) {
@@ -276,6 +327,34 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   }
 }
 
+// out[t, h, map, :] from the nsplit partial results of a decoded token's
+// head. One wave per (token, head * kmaps + map).
+__global__ void merge_splits_kernel(float* __restrict__ out,
+                                    const float* __restrict__ partial,
+                                    const int* __restrict__ tok_seq,
+                                    const int* __restrict__ seq_len,
+                                    int HM, int nsplit, int dv) {
+  const int t = blockIdx.x, hm = blockIdx.y, lane = threadIdx.x;
+  if (seq_len[tok_seq[t]] == 0) return;  // padding row
+  const float* p = partial + ((int64_t)t * HM + hm) * nsplit * (dv + 2);
+  float mx = -INFINITY;
+  for (int z = 0; z < nsplit; z++) mx = fmaxf(mx, p[z * (dv + 2)]);
+  float lt = 0.f;
+  for (int z = 0; z < nsplit; z++) {
+    const float mz = p[z * (dv + 2)];
+    if (mz != -INFINITY) lt += expf(mz - mx) * p[z * (dv + 2) + 1];
+  }
+  const float inv = 1.f / lt;
+  for (int ch = lane; ch < dv; ch += 64) {
+    float o = 0.f;
+    for (int z = 0; z < nsplit; z++) {
+      const float mz = p[z * (dv + 2)];
+      if (mz != -INFINITY) o += expf(mz - mx) * p[z * (dv + 2) + 2 + ch];
+    }
+    out[((int64_t)t * HM + hm) * dv + ch] = o * inv;
+  }
+}
+
 inline size_t lds_bytes(int KC, int DN) {
   const int KCH = KC < 4 ? KC : 4, DCH = DN < 8 ? DN : 8;
   return (size_t)(BN * (KCH * 32 + PADE) + DCH * 16 * (BN + PADE) +
@@ -284,8 +363,15 @@ inline size_t lds_bytes(int KC, int DN) {
 
 template <int KC, int DN, typename TO>
 void launch(dim3 grid, TO* out, const MfmaArgs& a) {
-  hipLaunchKernelGGL((paged_attention_mfma_kernel<KC, DN, TO>), grid, dim3(256),
-                     lds_bytes(KC, DN), cur_stream(), out, a);
+  if (a.partial) {
+    if constexpr (std::is_same<TO, float>::value)
+      hipLaunchKernelGGL((paged_attention_mfma_kernel<KC, DN, float, true>),
+                         grid, dim3(256), lds_bytes(KC, DN), cur_stream(), out,
+                         a);
+  } else {
+    hipLaunchKernelGGL((paged_attention_mfma_kernel<KC, DN, TO, false>), grid,
+                       dim3(256), lds_bytes(KC, DN), cur_stream(), out, a);
+  }
 }
 
 // padded sizes the kernel is built for: key chunks of 32, value chunks of 16
@@ -414,11 +500,95 @@ void paged_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
   a.scale = (float)scale; a.temp_coef = (float)temp_coef;
   a.temp_every = (int)temp_every; a.has_bias = r1 ? 1 : 0;
   a.kmaps = (int)kmaps; a.krow = krow; a.vrow = vrow; a.window = (int)window;
+  a.seq_len = nullptr; a.nsplit = 1; a.partial = nullptr;
   const int KC = pick_kc(dk), DN = pick_dn(dv);
   const dim3 grid(NT, H * kmaps);
   const bool ok = f32out ? dispatch<float>(KC, DN, grid, ptr<float>(out), a)
                          : dispatch<bf16_t>(KC, DN, grid, ptr<bf16_t>(out), a);
   TORCH_CHECK(ok, "seqmix: mfma attention sizes");
+}
+
+// Decoded tokens (one row each, rows [0, T) of out/proj): the query heads
+// that share a kv head form the rows of a matrix-core tile and the keys of
+// a token are split over `nsplit` workgroups. out [T, H, kmaps, dv] fp32;
+// partial is scratch [T, H, kmaps, nsplit, dv + 2] fp32.
+void paged_attention_mfma_decode(torch::Tensor out, torch::Tensor partial,
+                                 torch::Tensor proj, int64_t off_q,
+                                 torch::Tensor kcache,
+                                 c10::optional<torch::Tensor> vcache,
+                                 torch::Tensor page_table,
+                                 torch::Tensor tok_seq, torch::Tensor positions,
+                                 torch::Tensor seq_len, double scale,
+                                 int64_t kmaps, int64_t window) {
+  SEQ_CHECK(out.dim() == 4 && out.is_contiguous() && out.size(2) == kmaps &&
+                out.scalar_type() == torch::kFloat,
+            "mfma decode out [T, H, maps, dv] fp32");
+  const int T_ = out.size(0), H = out.size(1), dv = out.size(3);
+  const int G = kcache.size(1), ps = kcache.size(2), krow = kcache.size(3);
+  SEQ_CHECK(kmaps >= 1 && krow % kmaps == 0 && window >= 0, "key maps/window");
+  const int dk = krow / kmaps;
+  SEQ_CHECK(partial.dim() == 5 && partial.is_contiguous() &&
+                partial.scalar_type() == torch::kFloat &&
+                partial.size(0) == T_ && partial.size(1) == H &&
+                partial.size(2) == kmaps && partial.size(3) >= 1 &&
+                partial.size(4) == dv + 2, "mfma decode scratch");
+  const int nsplit = partial.size(3);
+  SEQ_CHECK(proj.scalar_type() == torch::kBFloat16 &&
+                kcache.scalar_type() == torch::kBFloat16 &&
+                kcache.is_contiguous() && G >= 1 && H % G == 0,
+            "mfma attention is bf16");
+  const bf16_t* vptr;
+  int vrow;
+  if (vcache) {
+    SEQ_CHECK(vcache->scalar_type() == torch::kBFloat16 &&
+                  vcache->is_contiguous() && vcache->size(3) == dv &&
+                  vcache->size(1) == G && vcache->size(2) == ps &&
+                  vcache->size(0) == kcache.size(0), "mfma value cache");
+    vptr = cptr<bf16_t>(*vcache);
+    vrow = dv;
+  } else {
+    SEQ_CHECK(dv <= krow, "values inside the key rows");
+    vptr = cptr<bf16_t>(kcache);
+    vrow = krow;
+  }
+  SEQ_CHECK(paged_attention_mfma_supported(dk, dv, true), "mfma attention sizes");
+  SEQ_CHECK(reinterpret_cast<uintptr_t>(kcache.data_ptr()) % 16 == 0 &&
+                reinterpret_cast<uintptr_t>(vptr) % 16 == 0 && krow % 8 == 0 &&
+                vrow % 8 == 0, "mfma attention cache alignment");
+  SEQ_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(0) >= T_ &&
+                off_q >= 0 && off_q + H * kmaps * dk <= proj.size(1),
+            "mfma attention q");
+  SEQ_CHECK(page_table.scalar_type() == torch::kInt && page_table.dim() == 2 &&
+                page_table.stride(1) == 1, "page table");
+  for (const torch::Tensor* t : {&tok_seq, &positions})
+    SEQ_CHECK(t->scalar_type() == torch::kInt && t->is_contiguous() &&
+                  t->numel() >= T_, "token descriptors");
+  SEQ_CHECK(seq_len.scalar_type() == torch::kInt && seq_len.is_contiguous() &&
+                seq_len.numel() <= page_table.size(0), "seq_len");
+  if (T_ == 0) return;
+  MfmaArgs a;
+  a.proj = cptr<bf16_t>(proj); a.proj_stride = (int)proj.stride(0);
+  a.off_q = (int)off_q;
+  a.kcache = cptr<bf16_t>(kcache); a.vcache = vptr;
+  a.page_table = cptr<int>(page_table);
+  a.table_stride = (int)page_table.stride(0);
+  a.tile_row0 = nullptr; a.tile_rows = nullptr;
+  a.tok_seq = cptr<int>(tok_seq); a.positions = cptr<int>(positions);
+  a.r1 = nullptr; a.r2 = nullptr;
+  a.H = H; a.G = G; a.dk = dk; a.dv = dv; a.ps = ps;
+  a.scale = (float)scale; a.temp_coef = 0.f; a.temp_every = 1; a.has_bias = 0;
+  a.kmaps = (int)kmaps; a.krow = krow; a.vrow = vrow; a.window = (int)window;
+  a.seq_len = cptr<int>(seq_len); a.nsplit = nsplit;
+  a.partial = ptr<float>(partial);
+  const int KC = pick_kc(dk), DN = pick_dn(dv);
+  const int gsz = H / G, nhb = (gsz + 63) / 64;
+  const dim3 grid(T_, G * kmaps * nhb, nsplit);
+  TORCH_CHECK(dispatch<float>(KC, DN, grid, ptr<float>(out), a),
+              "seqmix: mfma attention sizes");
+  hipLaunchKernelGGL(merge_splits_kernel, dim3(T_, H * kmaps), dim3(64), 0,
+                     cur_stream(), ptr<float>(out), cptr<float>(partial),
+                     cptr<int>(tok_seq), cptr<int>(seq_len), H * (int)kmaps,
+                     nsplit, dv);
 }
 
 void biased_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,

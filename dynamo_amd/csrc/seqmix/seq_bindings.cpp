@@ -66,7 +66,8 @@ void diff_norm_gate(Tensor out, Tensor a, Tensor lambda, double post,
 void head_sigmoid_scale(Tensor out, Tensor x, Tensor gate);
 void rglru_scan(Tensor out, Tensor u, Tensor gates, Tensor br, Tensor bi,
                 Tensor lam, Tensor y, Tensor state, Tensor seq_start,
-                Tensor seq_len, Tensor seq_slot, Tensor seq_pos0, double decay);
+                Tensor seq_len, Tensor seq_slot, Tensor seq_pos0, double decay,
+                int64_t max_len);
 bool biased_attention_mfma_supported(int64_t dk, int64_t dv);
 bool paged_attention_mfma_supported(int64_t dk, int64_t dv, bool f32out);
 void paged_attention_mfma(Tensor out, Tensor proj, int64_t off_q, Tensor kcache,
@@ -81,6 +82,12 @@ void biased_attention_mfma(Tensor out, Tensor proj, int64_t off_q,
                            int64_t max_tile_rows, Tensor tok_seq,
                            Tensor positions, OptTensor r1, OptTensor r2,
                            double scale, double temp_coef, int64_t temp_every);
+
+void paged_attention_mfma_decode(Tensor out, Tensor partial, Tensor proj,
+                                 int64_t off_q, Tensor kcache, OptTensor vcache,
+                                 Tensor page_table, Tensor tok_seq,
+                                 Tensor positions, Tensor seq_len, double scale,
+                                 int64_t kmaps, int64_t window);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "dynamo_amd sequence-mixer kernels (gfx950)";
@@ -110,4 +117,5 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("biased_attention_mfma", &biased_attention_mfma);
   m.def("paged_attention_mfma_supported", &paged_attention_mfma_supported);
   m.def("paged_attention_mfma", &paged_attention_mfma);
+  m.def("paged_attention_mfma_decode", &paged_attention_mfma_decode);
 }

@@ -18,7 +18,79 @@ inline int row_block(int W) {
 //   delta given:  res += mult * LN(delta) * post_w   (post_w absent: += delta)
 //   out given:    out = LN(res) * w
 // LN(x) = (x - mean) / sqrt(var + eps), var = mean of squared deviations
-// (two passes, so a large mean does not cancel).
+// (two passes, so a large mean does not cancel). A thread keeps its NI
+// entries of the row in registers, so delta and res are read once and res
+// and out written once; rows wider than NI * blockDim take the looping
+// kernel below.
+template <typename T, int NI>
+__global__ void residual_layernorm_reg_kernel(
+    T* __restrict__ out, float* __restrict__ res, const T* __restrict__ delta,
+    const float* __restrict__ post_w, float mult, const float* __restrict__ w,
+    float eps, int W) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  float* r = res + (int64_t)t * W;
+  float x[NI];
+#pragma unroll
+  for (int k = 0; k < NI; k++) {
+    const int i = threadIdx.x + k * blockDim.x;
+    x[k] = i < W ? r[i] : 0.f;
+  }
+  if (delta) {
+    const T* dl = delta + (int64_t)t * W;
+    float d[NI];
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < NI; k++) {
+      const int i = threadIdx.x + k * blockDim.x;
+      d[k] = i < W ? to_f(dl[i]) : 0.f;
+      s += d[k];
+    }
+    if (post_w) {
+      const float mean = block_sum(s, scratch) / (float)W;
+      float ss = 0.f;
+#pragma unroll
+      for (int k = 0; k < NI; k++) {
+        const int i = threadIdx.x + k * blockDim.x;
+        const float c = i < W ? d[k] - mean : 0.f;
+        ss += c * c;
+      }
+      const float inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)W + eps);
+#pragma unroll
+      for (int k = 0; k < NI; k++) {
+        const int i = threadIdx.x + k * blockDim.x;
+        if (i < W) x[k] += mult * ((d[k] - mean) * inv * post_w[i]);
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < NI; k++) x[k] += d[k];
+    }
+#pragma unroll
+    for (int k = 0; k < NI; k++) {
+      const int i = threadIdx.x + k * blockDim.x;
+      if (i < W) r[i] = x[k];
+    }
+  }
+  if (!out) return;
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NI; k++) s += x[k];  // entries past W are 0
+  const float mean = block_sum(s, scratch) / (float)W;
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NI; k++) {
+    const int i = threadIdx.x + k * blockDim.x;
+    const float c = i < W ? x[k] - mean : 0.f;
+    ss += c * c;
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)W + eps);
+#pragma unroll
+  for (int k = 0; k < NI; k++) {
+    const int i = threadIdx.x + k * blockDim.x;
+    if (i < W) out[(int64_t)t * W + i] = from_f<T>((x[k] - mean) * inv * w[i]);
+  }
+}
+
 template <typename T>
 __global__ void residual_layernorm_kernel(
     T* __restrict__ out, float* __restrict__ res, const T* __restrict__ delta,
@@ -61,16 +133,34 @@ __global__ void residual_layernorm_kernel(
 }
 
 // xIELU: z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (e^z - 1 - z) + z/2
+DEVINL float xielu_f(float z, float ap, float aq) {
+  return z > 0.f ? ap * z * z + 0.5f * z : aq * (expm1f(z) - z) + 0.5f * z;
+}
+
+// 16 bytes per thread and step; n is a multiple of 16 / sizeof(T)
+template <typename T>
+__global__ void xielu_vec_kernel(T* __restrict__ out, const T* __restrict__ x,
+                                 const float* __restrict__ pq, int64_t nvec) {
+  constexpr int N = 16 / sizeof(T);
+  const float ap = softplus_f(pq[0]), aq = 0.5f + softplus_f(pq[1]);
+  union V { uint4 raw; T e[N]; };
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    V v, o;
+    v.raw = reinterpret_cast<const uint4*>(x)[i];
+#pragma unroll
+    for (int k = 0; k < N; k++) o.e[k] = from_f<T>(xielu_f(to_f(v.e[k]), ap, aq));
+    reinterpret_cast<uint4*>(out)[i] = o.raw;
+  }
+}
+
 template <typename T>
 __global__ void xielu_kernel(T* __restrict__ out, const T* __restrict__ x,
                              const float* __restrict__ pq, int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const float ap = softplus_f(pq[0]), aq = 0.5f + softplus_f(pq[1]);
-  const float z = to_f(x[i]);
-  const float y = z > 0.f ? ap * z * z + 0.5f * z
-                          : aq * (expm1f(z) - z) + 0.5f * z;
-  out[i] = from_f<T>(y);
+  out[i] = from_f<T>(xielu_f(to_f(x[i]), ap, aq));
 }
 
 // Rotation of one pair at angle pos * freq. fp32 throughout.
@@ -202,40 +292,132 @@ DEVINL float gelu_tanh_f(float z) {
 //   r = sigmoid(gr + br), i = sigmoid(gi + bi), a = exp(-decay * r * softplus(lam))
 //   S <- a S + sqrt(1 - a^2) * i * u ;   out = S * gelu_tanh(y)
 // gates [nb, T, 2 bw] fp32 hold gr (first bw) and gi of each block's
-// channels. A thread owns one channel of one sequence and walks the
-// sequence's rows of this step; the slot's state continues earlier steps
-// and a sequence at position 0 starts from S = 0.
+// channels. The slot's state continues earlier steps and a sequence at
+// position 0 starts from S = 0.
+//
+// The recurrence is linear in S, so a long portion is cut into chunks of
+// `chunk` tokens that run in parallel: a first kernel reduces every chunk
+// but the last to (A, B) with S_end = A S_begin + B, and the scan kernel
+// of chunk k first folds the summaries of chunks 0..k-1 onto the slot's
+// state. A thread owns one channel of one chunk of one sequence. Decoded
+// tokens and short portions are a single chunk and skip the first kernel.
+struct RglruCoef {
+  float a, b;
+};
+DEVINL RglruCoef rglru_coef(float gr, float gi, float cbr, float cbi,
+                            float rate, float u) {
+  const float r = sigmoid_f(gr + cbr);
+  const float ig = sigmoid_f(gi + cbi);
+  const float la = rate * r;
+  RglruCoef c;
+  c.a = expf(la);
+  // 1 - a^2 = -expm1(2 log a): exact also where a is close to 1
+  c.b = sqrtf(-expm1f(2.f * la)) * (ig * u);
+  return c;
+}
+
+__global__ void rglru_chunk_summary_kernel(
+    float* __restrict__ sumA, float* __restrict__ sumB,  // [B, nch, C]
+    const float* __restrict__ u, const float* __restrict__ gates,
+    const float* __restrict__ br, const float* __restrict__ bi,
+    const float* __restrict__ lam, const int* __restrict__ seq_start,
+    const int* __restrict__ seq_len, int Ttot, int C, int bw, float decay,
+    int chunk, int nch) {
+  const int s = blockIdx.z, k = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int len = seq_len[s];
+  // the last chunk of a sequence carries into nothing
+  if (c >= C || (k + 1) * chunk >= len) return;
+  const int start = seq_start[s] + k * chunk;
+  const int b = c / bw, o = c - b * bw;
+  const float* gr = gates + ((int64_t)b * Ttot + start) * 2 * bw + o;
+  const float rate = -decay * softplus_f(lam[c]);
+  const float cbr = br[c], cbi = bi[c];
+  float A = 1.f, S = 0.f;
+#pragma unroll 4
+  for (int j = 0; j < chunk; j++) {
+    const RglruCoef q = rglru_coef(gr[(int64_t)j * 2 * bw],
+                                   gr[(int64_t)j * 2 * bw + bw], cbr, cbi, rate,
+                                   u[(int64_t)(start + j) * C + c]);
+    A *= q.a;
+    S = q.a * S + q.b;
+  }
+  sumA[((int64_t)s * nch + k) * C + c] = A;
+  sumB[((int64_t)s * nch + k) * C + c] = S;
+}
+
 template <typename T>
 __global__ void rglru_scan_kernel(
     T* __restrict__ out, const float* __restrict__ u,
     const float* __restrict__ gates, const float* __restrict__ br,
     const float* __restrict__ bi, const float* __restrict__ lam,
     const T* __restrict__ y, int y_stride, float* __restrict__ state,
+    const float* __restrict__ sumA, const float* __restrict__ sumB,
     const int* __restrict__ seq_start, const int* __restrict__ seq_len,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_pos0,
-    int Ttot, int C, int bw, float decay) {
-  const int s = blockIdx.y;
+    int Ttot, int C, int bw, float decay, int chunk, int nch) {
+  const int s = blockIdx.z, k = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   const int len = seq_len[s];
-  if (c >= C || len == 0) return;
-  const int start = seq_start[s];
+  if (c >= C || k * chunk >= len) return;
+  const int n = min(chunk, len - k * chunk);
+  const int start = seq_start[s] + k * chunk;
   float* st = state + (int64_t)seq_slot[s] * C + c;
   float S = seq_pos0[s] > 0 ? *st : 0.f;
+  for (int kk = 0; kk < k; kk++)
+    S = sumA[((int64_t)s * nch + kk) * C + c] * S +
+        sumB[((int64_t)s * nch + kk) * C + c];
   const int b = c / bw, o = c - b * bw;
   const float* gr = gates + ((int64_t)b * Ttot + start) * 2 * bw + o;
   const float rate = -decay * softplus_f(lam[c]);
   const float cbr = br[c], cbi = bi[c];
 #pragma unroll 4
-  for (int k = 0; k < len; k++) {
-    const int64_t t = start + k;
-    const float r = sigmoid_f(gr[(int64_t)k * 2 * bw] + cbr);
-    const float ig = sigmoid_f(gr[(int64_t)k * 2 * bw + bw] + cbi);
-    const float la = rate * r;
-    const float a = expf(la);
-    // 1 - a^2 = -expm1(2 log a): exact also where a is close to 1
-    const float mul = sqrtf(-expm1f(2.f * la));
-    S = a * S + mul * (ig * u[t * C + c]);
+  for (int j = 0; j < n; j++) {
+    const int64_t t = start + j;
+    const RglruCoef q = rglru_coef(gr[(int64_t)j * 2 * bw],
+                                   gr[(int64_t)j * 2 * bw + bw], cbr, cbi, rate,
+                                   u[t * C + c]);
+    S = q.a * S + q.b;
     out[t * C + c] = from_f<T>(S * gelu_tanh_f(to_f(y[t * y_stride + c])));
+  }
+  // the state is read by every chunk of the sequence before any write can
+  // land only if the last chunk is alone; otherwise the earlier chunks read
+  // the slot in this same launch, so the last chunk writes it in a second
+  // launch (see rglru_state_kernel)
+  if (nch == 1) *st = S;
+}
+
+// The state after the last token of each multi-chunk sequence: fold every
+// chunk summary but the last onto the old state, then walk the last chunk.
+__global__ void rglru_state_kernel(
+    float* __restrict__ state, const float* __restrict__ u,
+    const float* __restrict__ gates, const float* __restrict__ br,
+    const float* __restrict__ bi, const float* __restrict__ lam,
+    const float* __restrict__ sumA, const float* __restrict__ sumB,
+    const int* __restrict__ seq_start, const int* __restrict__ seq_len,
+    const int* __restrict__ seq_slot, const int* __restrict__ seq_pos0,
+    int Ttot, int C, int bw, float decay, int chunk, int nch) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int len = seq_len[s];
+  if (c >= C || len == 0) return;
+  float* st = state + (int64_t)seq_slot[s] * C + c;
+  float S = seq_pos0[s] > 0 ? *st : 0.f;
+  const int last = (len - 1) / chunk;
+  for (int kk = 0; kk < last; kk++)
+    S = sumA[((int64_t)s * nch + kk) * C + c] * S +
+        sumB[((int64_t)s * nch + kk) * C + c];
+  const int start = seq_start[s] + last * chunk;
+  const int n = len - last * chunk;
+  const int b = c / bw, o = c - b * bw;
+  const float* gr = gates + ((int64_t)b * Ttot + start) * 2 * bw + o;
+  const float rate = -decay * softplus_f(lam[c]);
+  const float cbr = br[c], cbi = bi[c];
+  for (int j = 0; j < n; j++) {
+    const RglruCoef q = rglru_coef(gr[(int64_t)j * 2 * bw],
+                                   gr[(int64_t)j * 2 * bw + bw], cbr, cbi, rate,
+                                   u[(int64_t)(start + j) * C + c]);
+    S = q.a * S + q.b;
   }
   *st = S;
 }
@@ -271,12 +453,33 @@ void residual_layernorm(c10::optional<torch::Tensor> out, torch::Tensor res,
               "post-norm weight");
   if (T_ == 0) return;
   const torch::Tensor& ty = out ? *out : *delta;
-  DISPATCH_ACT(ty, hipLaunchKernelGGL(
-      residual_layernorm_kernel<T>, dim3(T_), dim3(row_block(W)), 0,
-      cur_stream(), out ? ptr<T>(*out) : (T*)nullptr, ptr<float>(res),
-      delta ? cptr<T>(*delta) : (const T*)nullptr,
-      post_w ? cptr<float>(*post_w) : (const float*)nullptr, (float)mult,
-      w ? cptr<float>(*w) : (const float*)nullptr, (float)eps, W););
+  // 256 threads with up to 8 entries each in registers (many rows), or up
+  // to 1024 threads with 2-4 entries each (few rows: decoding, where the
+  // row's latency counts); wider rows loop
+  const int threads = W <= 512 ? row_block((W + 3) / 4)
+                      : T_ <= 1024 ? std::min(1024, row_block((W + 1) / 2))
+                                   : 256;
+  const int ni = (W + threads - 1) / threads;
+#define LN_ARGS                                                               \
+  out ? ptr<T>(*out) : (T*)nullptr, ptr<float>(res),                          \
+      delta ? cptr<T>(*delta) : (const T*)nullptr,                            \
+      post_w ? cptr<float>(*post_w) : (const float*)nullptr, (float)mult,     \
+      w ? cptr<float>(*w) : (const float*)nullptr, (float)eps, W
+  DISPATCH_ACT(ty, {
+    if (ni <= 4)
+      hipLaunchKernelGGL((residual_layernorm_reg_kernel<T, 4>), dim3(T_),
+                         dim3(threads), 0, cur_stream(), LN_ARGS);
+    else if (ni <= 8)
+      hipLaunchKernelGGL((residual_layernorm_reg_kernel<T, 8>), dim3(T_),
+                         dim3(threads), 0, cur_stream(), LN_ARGS);
+    else if (ni <= 16)
+      hipLaunchKernelGGL((residual_layernorm_reg_kernel<T, 16>), dim3(T_),
+                         dim3(threads), 0, cur_stream(), LN_ARGS);
+    else
+      hipLaunchKernelGGL(residual_layernorm_kernel<T>, dim3(T_), dim3(1024), 0,
+                         cur_stream(), LN_ARGS);
+  });
+#undef LN_ARGS
 }
 
 void xielu(torch::Tensor out, torch::Tensor x, torch::Tensor pq) {
@@ -287,9 +490,22 @@ void xielu(torch::Tensor out, torch::Tensor x, torch::Tensor pq) {
                 pq.numel() == 2, "xielu parameters");
   const int64_t n = x.numel();
   if (n == 0) return;
-  DISPATCH_ACT(x, hipLaunchKernelGGL(
-      xielu_kernel<T>, dim3((n + 255) / 256), dim3(256), 0, cur_stream(),
-      ptr<T>(out), cptr<T>(x), cptr<float>(pq), n););
+  const bool vec = reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0 &&
+                   (n * x.element_size()) % 16 == 0;
+  DISPATCH_ACT(x, {
+    if (vec) {
+      const int64_t nvec = n * sizeof(T) / 16;
+      const int64_t blocks = std::min<int64_t>((nvec + 255) / 256, 8192);
+      hipLaunchKernelGGL(xielu_vec_kernel<T>, dim3(blocks), dim3(256), 0,
+                         cur_stream(), ptr<T>(out), cptr<T>(x),
+                         cptr<float>(pq), nvec);
+    } else {
+      hipLaunchKernelGGL(xielu_kernel<T>, dim3((n + 255) / 256), dim3(256), 0,
+                         cur_stream(), ptr<T>(out), cptr<T>(x),
+                         cptr<float>(pq), n);
+    }
+  });
 }
 
 void rope_rows(torch::Tensor dst, int64_t dst_col, int64_t dst_vec,
@@ -397,7 +613,8 @@ void rglru_scan(torch::Tensor out, torch::Tensor u, torch::Tensor gates,
                 torch::Tensor br, torch::Tensor bi, torch::Tensor lam,
                 torch::Tensor y, torch::Tensor state, torch::Tensor seq_start,
                 torch::Tensor seq_len, torch::Tensor seq_slot,
-                torch::Tensor seq_pos0, double decay) {
+                torch::Tensor seq_pos0, double decay, int64_t max_len) {
+  // max_len: an upper bound of the longest sequence portion of this step
   const int T_ = u.size(0), C = u.size(1);
   const int B = seq_start.size(0);
   SEQ_CHECK(u.dim() == 2 && u.scalar_type() == torch::kFloat &&
@@ -419,13 +636,38 @@ void rglru_scan(torch::Tensor out, torch::Tensor u, torch::Tensor gates,
   check_seq(seq_len, B, "seq_len");
   check_seq(seq_slot, B, "seq_slot");
   check_seq(seq_pos0, B, "seq_pos0");
+  SEQ_CHECK(max_len >= 1, "longest portion");
   if (T_ == 0 || B == 0) return;
   const int threads = 64;
+  const int chunk = 64;
+  const int nch = (int)((std::min<int64_t>(max_len, T_) + chunk - 1) / chunk);
+  const int cb = (C + threads - 1) / threads;
+  torch::Tensor sums;
+  const float* sumA = nullptr;
+  const float* sumB = nullptr;
+  if (nch > 1) {
+    sums = torch::empty({2, B, nch, C}, u.options());
+    sumA = cptr<float>(sums);
+    sumB = sumA + (int64_t)B * nch * C;
+    hipLaunchKernelGGL(rglru_chunk_summary_kernel, dim3(cb, nch, B),
+                       dim3(threads), 0, cur_stream(), ptr<float>(sums),
+                       ptr<float>(sums) + (int64_t)B * nch * C, cptr<float>(u),
+                       cptr<float>(gates), cptr<float>(br), cptr<float>(bi),
+                       cptr<float>(lam), cptr<int>(seq_start),
+                       cptr<int>(seq_len), T_, C, bw, (float)decay, chunk, nch);
+  }
   DISPATCH_ACT(y, hipLaunchKernelGGL(
-      rglru_scan_kernel<T>, dim3((C + threads - 1) / threads, B), dim3(threads),
-      0, cur_stream(), ptr<T>(out), cptr<float>(u), cptr<float>(gates),
-      cptr<float>(br), cptr<float>(bi), cptr<float>(lam), cptr<T>(y),
-      (int)y.stride(0), ptr<float>(state), cptr<int>(seq_start),
-      cptr<int>(seq_len), cptr<int>(seq_slot), cptr<int>(seq_pos0), T_, C, bw,
-      (float)decay););
+      rglru_scan_kernel<T>, dim3(cb, nch, B), dim3(threads), 0, cur_stream(),
+      ptr<T>(out), cptr<float>(u), cptr<float>(gates), cptr<float>(br),
+      cptr<float>(bi), cptr<float>(lam), cptr<T>(y), (int)y.stride(0),
+      ptr<float>(state), sumA, sumB, cptr<int>(seq_start), cptr<int>(seq_len),
+      cptr<int>(seq_slot), cptr<int>(seq_pos0), T_, C, bw, (float)decay, chunk,
+      nch););
+  if (nch > 1)
+    hipLaunchKernelGGL(rglru_state_kernel, dim3(cb, B), dim3(threads), 0,
+                       cur_stream(), ptr<float>(state), cptr<float>(u),
+                       cptr<float>(gates), cptr<float>(br), cptr<float>(bi),
+                       cptr<float>(lam), sumA, sumB, cptr<int>(seq_start),
+                       cptr<int>(seq_len), cptr<int>(seq_slot),
+                       cptr<int>(seq_pos0), T_, C, bw, (float)decay, chunk, nch);
 }

@@ -64,7 +64,8 @@ class GraphRunner:
             meta.seq_batch = SeqBatch(
                 tok_seq=self.seq_rows[:bc], seq_start=self.seq_rows[:bc],
                 seq_len=self.seq_len[:bc], seq_slot=self.seq_slot[:bc],
-                seq_pos0=self.positions[:bc], page_table=self.page_table[:bc])
+                seq_pos0=self.positions[:bc], page_table=self.page_table[:bc],
+                num_decode=bc)
             meta.state_pool = self.runner.state_pool
         return meta
 

@@ -301,19 +301,34 @@ def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
         out = torch.empty(T, H, kmaps, dv, dtype=torch.float32,
                           device=q.device)
         m = hip_seq()
-        # prompt portions in bf16 go to the MFMA kernel when the row sizes
-        # fit it; decoded tokens, fp32 and other sizes take the row kernel
-        krow = kcache.shape[3]
-        tiled = (sb.tiles is not None and q.dtype == torch.bfloat16
-                 and m.paged_attention_mfma_supported(krow // kmaps, dv, True)
-                 and krow % 8 == 0 and kcache.data_ptr() % 16 == 0
-                 and (vcache is None or vcache.data_ptr() % 16 == 0))
-        nrow = sb.num_decode if tiled else T
-        if nrow:
+        # bf16 rows whose sizes fit go to the matrix cores: prompt portions
+        # as 64-row tiles, decoded tokens (rows [0, num_decode)) with their
+        # heads as tile rows when at least 8 heads share a kv head. fp32,
+        # other sizes and the remaining rows take the row kernel.
+        krow, G = kcache.shape[3], kcache.shape[1]
+        fits = (q.dtype == torch.bfloat16
+                and m.paged_attention_mfma_supported(krow // kmaps, dv, True)
+                and krow % 8 == 0 and kcache.data_ptr() % 16 == 0
+                and (vcache is None or vcache.data_ptr() % 16 == 0))
+        tiled = fits and sb.tiles is not None
+        ndec = min(sb.num_decode, T)
+        done = 0
+        if fits and ndec and H // G >= 8:
+            nsplit = max(1, min(16, 512 // (ndec * G * kmaps)))
+            part = torch.empty(ndec, H, kmaps, nsplit, dv + 2,
+                               dtype=torch.float32, device=q.device)
+            m.paged_attention_mfma_decode(
+                out[:ndec], part, q[:ndec], off_q, kcache, vcache,
+                sb.page_table, sb.tok_seq[:ndec], positions[:ndec],
+                sb.seq_len, float(scale), int(kmaps), int(window))
+            done = ndec
+        end = ndec if tiled else T
+        if end > done:
             m.paged_attention_rows(
-                out[:nrow], q[:nrow], off_q, kcache, vcache, sb.page_table,
-                sb.tok_seq[:nrow], positions[:nrow], sb.seq_len, None, None,
-                float(scale), 0.0, 1, int(kmaps), int(window))
+                out[done:end], q[done:end], off_q, kcache, vcache,
+                sb.page_table, sb.tok_seq[done:end], positions[done:end],
+                sb.seq_len, None, None, float(scale), 0.0, 1, int(kmaps),
+                int(window))
         if tiled and sb.tiles[0].numel():
             m.paged_attention_mfma(
                 out, q, off_q, kcache, vcache, sb.page_table, sb.tiles[0],
@@ -363,8 +378,12 @@ def rglru_scan(u, gates, br, bi, lam, y, state, sb: SeqBatch, decay: float,
     pre-activations gates [nb, T, 2*bw]; returns S * gelu_tanh(y[:, :C])."""
     if u.is_cuda:
         out = torch.empty(u.shape, dtype=out_dtype, device=u.device)
+        # long portions are scanned in parallel chunks; the kernel needs an
+        # upper bound of the longest portion (known on the host, or all rows)
+        longest = (max((n for _s, n, _l, _p in sb.host), default=1)
+                   if sb.host is not None else u.shape[0])
         hip_seq().rglru_scan(out, u, gates, br, bi, lam, y, state, *_args(sb),
-                             float(decay))
+                             float(decay), max(1, int(longest)))
         return out
     return seq_ref.rglru_scan(u, gates, br, bi, lam, y, state, sb, decay,
                               out_dtype)

@@ -544,6 +544,54 @@ def test_mfma_prompt_attention_matches_row_kernel(H, G, dk, dv, kmaps, window,
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("H,G,dk,dv,kmaps,window,alias", [
+    (16, 1, 576, 512, 1, 0, True),      # latent rows, 16 heads on one row
+    (5, 1, 192, 128, 1, 0, True),       # fewer heads than a tile has rows
+    (80, 1, 64, 64, 1, 0, False),       # more heads than one tile (64 + 16)
+    (16, 2, 64, 128, 2, 100, False),    # differential heads, 8 per kv head
+])
+def test_mfma_decode_matches_row_kernel(H, G, dk, dv, kmaps, window, alias):
+    """Single decoded tokens of sequences of unequal length (one of them a
+    padding row, one a sequence of one token) with heads as tile rows and
+    the keys split over workgroups, against the row kernel."""
+    from dynamo_amd.ops import seq as sops
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(H + dk)
+    ps, krow = 16, kmaps * dk
+    ctx = [700, 1, 64, 65, 333, 129]
+    pad = 2                                  # this row's seq_len is 0
+    caches, tabs, base = [], [], 0
+    for n in ctx:
+        k = (torch.randn(n, G, krow, generator=g) * 0.6).to(torch.bfloat16)
+        v = None if alias else torch.randn(n, G, dv, generator=g).to(torch.bfloat16)
+        kc, vc, tab = _paged(k, v, ps, extra=1, seed=n)
+        caches.append((kc, vc))
+        tabs.append(tab + base)
+        base += kc.shape[0]
+    kc = torch.cat([c[0] for c in caches]).to(dev)
+    vc = None if alias else torch.cat([c[1] for c in caches]).to(dev)
+    B = len(ctx)
+    pt = torch.zeros(B, max(len(t) for t in tabs), dtype=torch.int32)
+    for i, t in enumerate(tabs):
+        pt[i, :len(t)] = t
+    q = (torch.randn(B, H * krow, generator=g) * 0.6).to(torch.bfloat16).to(dev)
+    rows = torch.arange(B, dtype=torch.int32, device=dev)
+    lens = torch.ones(B, dtype=torch.int32)
+    lens[pad] = 0
+    pos = torch.tensor([n - 1 for n in ctx], dtype=torch.int32, device=dev)
+    outs = []
+    for ndec in (0, B):                      # row kernel, then matrix cores
+        sb = sops.SeqBatch(rows, rows, lens.to(dev), rows, pos,
+                           page_table=pt.to(dev), num_decode=ndec)
+        o = sops.paged_attention_rows(q, 0, H, kmaps, kc, vc, dv, pos, sb,
+                                      0.09, window).cpu()
+        outs.append(torch.cat([o[:pad], o[pad + 1:]]))
+    assert torch.isfinite(outs[1]).all()
+    scale = float(outs[0].abs().max())
+    assert float((outs[0] - outs[1]).abs().max()) < 2e-3 * scale
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("window", [5, 64, 70])
 def test_window_edges_on_the_matrix_cores(window):
     """The dominating key just outside / just inside the window, bf16
