@@ -151,9 +151,70 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 #pragma unroll
   for (int d = 0; d < DN; d++) acc_o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  const int kstep = HEADS ? a.nsplit : 1;
-  for (int t0 = (kv_begin / BN + (HEADS ? (int)blockIdx.z : 0)) * BN;
-       t0 < kv_end; t0 += kstep * BN) {
+  // ---- staging through registers: the loads of the next chunk are issued
+  // before the products of the current one, so their latency hides behind
+  // the matrix cores. One buffer serves key and value chunks in turn.
+  constexpr int NSK = (BN * KCH * 4 + 255) / 256;  // 16-byte pieces / thread
+  constexpr int NSV = (BN * DCH * 2 + 255) / 256;
+  constexpr int NST = NSK > NSV ? NSK : NSV;
+  short8_t stage[NST];
+  // Loads are unconditional with clamped addresses (a branch around a load
+  // would make each wait for the one before); what lies past the end of
+  // the keys or of the row is zeroed when the piece is written to LDS.
+  auto load_k = [&](int t0, int cc) {
+    constexpr int kvecs = KCH * 4;  // 16-byte pieces per staged row
+#pragma unroll
+    for (int u = 0; u < NSK; u++) {
+      const int slot = threadIdx.x + u * 256;
+      const int row = slot / kvecs, v = slot - row * kvecs;
+      const int j = min(t0 + row, kv_end - 1);
+      const int ch = min((cc * KCH * 4 + v) * 8, dk - 8);
+      const int64_t page = table[j / ps];
+      stage[u] = *reinterpret_cast<const short8_t*>(
+          a.kcache + ((page * G + g) * ps + (j % ps)) * a.krow + koff + ch);
+    }
+  };
+  auto store_k = [&](int t0, int cc) {
+    constexpr int kvecs = KCH * 4;
+#pragma unroll
+    for (int u = 0; u < NSK; u++) {
+      const int slot = threadIdx.x + u * 256;
+      const int row = slot / kvecs, v = slot - row * kvecs;
+      const bool ok = t0 + row < kv_end && (cc * KCH * 4 + v) * 8 < dk;
+      *reinterpret_cast<short8_t*>(k_lds + row * KS + v * 8) =
+          ok ? stage[u] : short8_t{};
+    }
+  };
+  // consecutive threads take consecutive keys of one channel group, so the
+  // transposed 2-byte LDS writes fall in consecutive banks
+  auto load_v = [&](int t0, int vc) {
+#pragma unroll
+    for (int u = 0; u < NSV; u++) {
+      const int slot = threadIdx.x + u * 256;
+      const int v = slot / BN, row = slot - v * BN;
+      const int j = min(t0 + row, kv_end - 1);
+      const int ch = min((vc * DCH * 2 + v) * 8, dv - 8);
+      const int64_t page = table[j / ps];
+      stage[u] = *reinterpret_cast<const short8_t*>(
+          a.vcache + ((page * G + g) * ps + (j % ps)) * a.vrow + ch);
+    }
+  };
+  auto store_v = [&](int t0, int vc) {
+#pragma unroll
+    for (int u = 0; u < NSV; u++) {
+      const int slot = threadIdx.x + u * 256;
+      const int v = slot / BN, row = slot - v * BN;
+      const bool ok = t0 + row < kv_end && (vc * DCH * 2 + v) * 8 < dv;
+      const short8_t x = ok ? stage[u] : short8_t{};
+#pragma unroll
+      for (int e = 0; e < 8; e++) vt_lds[(v * 8 + e) * VS + row] = x[e];
+    }
+  };
+
+  const int kstep = (HEADS ? a.nsplit : 1) * BN;
+  const int t_first = (kv_begin / BN + (HEADS ? (int)blockIdx.z : 0)) * BN;
+  if (t_first < kv_end) load_k(t_first, 0);
+  for (int t0 = t_first; t0 < kv_end; t0 += kstep) {
     // ---- S = Q K^T over key-channel chunks: block n covers keys
     //      t0 + 16 n + lr
     f32x4_t s[4];
@@ -162,19 +223,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 #pragma unroll
     for (int cc = 0; cc < NKCH; cc++) {
       __syncthreads();  // the previous readers of k_lds are done
-      constexpr int kvecs = KCH * 4;  // 16-byte pieces per staged row
-      for (int slot = threadIdx.x; slot < BN * kvecs; slot += 256) {
-        const int row = slot / kvecs, v = slot - row * kvecs;
-        const int j = t0 + row;
-        const int ch = (cc * KCH * 4 + v) * 8;
-        short8_t x{};
-        if (j < kv_end && ch < dk) {
-          const int64_t page = table[j / ps];
-          x = *reinterpret_cast<const short8_t*>(
-              a.kcache + ((page * G + g) * ps + (j % ps)) * a.krow + koff + ch);
-        }
-        *reinterpret_cast<short8_t*>(k_lds + row * KS + v * 8) = x;
-      }
+      store_k(t0, cc);
+      if (cc + 1 < NKCH) load_k(t0, cc + 1);
+      else load_v(t0, 0);
       __syncthreads();
       if (active)
 #pragma unroll
@@ -250,22 +301,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 #pragma unroll
     for (int vc = 0; vc < NDCH; vc++) {
       if (vc) __syncthreads();  // the previous chunk's readers are done
-      // consecutive threads take consecutive keys of one channel group, so
-      // the transposed 2-byte LDS writes fall in consecutive banks
-      constexpr int vvecs = DCH * 2;
-      for (int slot = threadIdx.x; slot < BN * vvecs; slot += 256) {
-        const int v = slot / BN, row = slot - v * BN;
-        const int j = t0 + row;
-        const int ch = (vc * DCH * 2 + v) * 8;
-        short8_t x{};
-        if (j < kv_end && ch < dv) {
-          const int64_t page = table[j / ps];
-          x = *reinterpret_cast<const short8_t*>(
-              a.vcache + ((page * G + g) * ps + (j % ps)) * a.vrow + ch);
-        }
-#pragma unroll
-        for (int e = 0; e < 8; e++) vt_lds[(v * 8 + e) * VS + row] = x[e];
-      }
+      store_v(t0, vc);
+      if (vc + 1 < NDCH) load_v(t0, vc + 1);
+      else if (t0 + kstep < kv_end) load_k(t0 + kstep, 0);
       __syncthreads();
       if (active)
 #pragma unroll
@@ -327,30 +365,38 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   }
 }
 
-// out[t, h, map, :] from the nsplit partial results of a decoded token's
-// head. One wave per (token, head * kmaps + map).
+// out[t, h, map, :] from the nsplit (<= 16) partial results of a decoded
+// token's head. One workgroup per (token, head * kmaps + map); the split
+// weights exp(m_z - max) / sum are formed once, then threads own channels.
+constexpr int MAXSPLIT = 16;
 __global__ void merge_splits_kernel(float* __restrict__ out,
                                     const float* __restrict__ partial,
                                     const int* __restrict__ tok_seq,
                                     const int* __restrict__ seq_len,
                                     int HM, int nsplit, int dv) {
-  const int t = blockIdx.x, hm = blockIdx.y, lane = threadIdx.x;
+  const int t = blockIdx.x, hm = blockIdx.y;
   if (seq_len[tok_seq[t]] == 0) return;  // padding row
-  const float* p = partial + ((int64_t)t * HM + hm) * nsplit * (dv + 2);
+  const int rec = dv + 2;
+  const float* p = partial + ((int64_t)t * HM + hm) * nsplit * rec;
+  float w[MAXSPLIT];
   float mx = -INFINITY;
-  for (int z = 0; z < nsplit; z++) mx = fmaxf(mx, p[z * (dv + 2)]);
+#pragma unroll
+  for (int z = 0; z < MAXSPLIT; z++) {
+    w[z] = z < nsplit ? p[z * rec] : -INFINITY;
+    mx = fmaxf(mx, w[z]);
+  }
   float lt = 0.f;
-  for (int z = 0; z < nsplit; z++) {
-    const float mz = p[z * (dv + 2)];
-    if (mz != -INFINITY) lt += expf(mz - mx) * p[z * (dv + 2) + 1];
+#pragma unroll
+  for (int z = 0; z < MAXSPLIT; z++) {
+    w[z] = w[z] == -INFINITY ? 0.f : expf(w[z] - mx);
+    if (z < nsplit) lt += w[z] * p[z * rec + 1];
   }
   const float inv = 1.f / lt;
-  for (int ch = lane; ch < dv; ch += 64) {
+  for (int ch = threadIdx.x; ch < dv; ch += blockDim.x) {
     float o = 0.f;
-    for (int z = 0; z < nsplit; z++) {
-      const float mz = p[z * (dv + 2)];
-      if (mz != -INFINITY) o += expf(mz - mx) * p[z * (dv + 2) + 2 + ch];
-    }
+#pragma unroll
+    for (int z = 0; z < MAXSPLIT; z++)
+      if (z < nsplit) o += w[z] * p[z * rec + 2 + ch];
     out[((int64_t)t * HM + hm) * dv + ch] = o * inv;
   }
 }
@@ -585,7 +631,9 @@ void paged_attention_mfma_decode(torch::Tensor out, torch::Tensor partial,
   const dim3 grid(T_, G * kmaps * nhb, nsplit);
   TORCH_CHECK(dispatch<float>(KC, DN, grid, ptr<float>(out), a),
               "seqmix: mfma attention sizes");
-  hipLaunchKernelGGL(merge_splits_kernel, dim3(T_, H * kmaps), dim3(64), 0,
+  SEQ_CHECK(nsplit <= MAXSPLIT, "too many key splits");
+  hipLaunchKernelGGL(merge_splits_kernel, dim3(T_, H * kmaps),
+                     dim3(dv <= 64 ? 64 : (dv <= 128 ? 128 : 256)), 0,
                      cur_stream(), ptr<float>(out), cptr<float>(partial),
                      cptr<int>(tok_seq), cptr<int>(seq_len), H * (int)kmaps,
                      nsplit, dv);
