@@ -24,7 +24,7 @@
 
 namespace {
 
-constexpr int EVMAX = 8;  // value channels per lane: dv <= 512
+constexpr int EVMAX = 16;  // value channels per lane: dv <= 1024
 
 // Append this step's keys (raw) and values (each head divided by its root
 // mean square when vnorm is set) to the paged cache. One wave per
@@ -363,7 +363,7 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
                    vrow % 2 == 0 &&
                    reinterpret_cast<uintptr_t>(kcache.data_ptr()) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(vptr) % 8 == 0;
-  const bool small = dv <= 128;
+  const bool small = dv <= 128, mid = dv <= 512;
 #define LAUNCH_ATT(GS_, VEC_, EVT_)                                         \
   hipLaunchKernelGGL((biased_attention_kernel<T, TO, GS_, VEC_, EVT_>),     \
       dim3(T_, H * kmaps / GS_), dim3(NW * 64), lds, cur_stream(),          \
@@ -377,8 +377,10 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
 #define LAUNCH_GS(GS_)                                                      \
   do {                                                                      \
     if (vec && small) LAUNCH_ATT(GS_, true, 2);                             \
+    else if (vec && mid) LAUNCH_ATT(GS_, true, 8);                          \
     else if (vec) LAUNCH_ATT(GS_, true, EVMAX);                             \
     else if (small) LAUNCH_ATT(GS_, false, 2);                              \
+    else if (mid) LAUNCH_ATT(GS_, false, 8);                                \
     else LAUNCH_ATT(GS_, false, EVMAX);                                     \
   } while (0)
   if (GS == 4) LAUNCH_GS(4);

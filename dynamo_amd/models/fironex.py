@@ -48,8 +48,6 @@ def build_mixer(kind: str, m: dict, width: int, eps: float, init: _Init):
             width, m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"],
             m["diff"], m["rot"], (m.get("mask") or {}).get("size"), eps, init)
     if kind == "latent_attention":
-        if int(m["rot"]["dims"]) != int(m["rot_dim"]):
-            raise ValueError("latent attention rotates its whole rotated part")
         return LatentAttention(
             width, m["heads"], m["dim"], m["rot_dim"], m["vdim"],
             m["kv_rank"], m["scale"], m["rot"], eps, init,

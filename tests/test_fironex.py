@@ -412,6 +412,24 @@ def test_large_heads(tmp_path, device):
     _check(eng, cfg, W, toks, [[90], [70, 1]])
 
 
+@pytest.mark.parametrize("device", DEVICES)
+def test_wide_latent_partly_rotated(tmp_path, device):
+    """A latent wider than 512 (the widest value row of the matrix-core
+    kernel) whose rotated part is only half rotated."""
+    la = copy.deepcopy(U.LATENT)
+    la["mixer"].update(heads=2, dim=8, rot_dim=16, vdim=8, kv_rank=600,
+                       rot={"base": 300.0, "dims": 8})
+    lb = U.latent_from(0, heads=3, dim=8, vdim=16, mlp=False)
+    lb["mixer"].update(rot_dim=16, kv_rank=600, rot={"base": 300.0, "dims": 8})
+    path, cfg, W = _case(tmp_path, [la, lb], seed=23, width=48, vocab=61)
+    toks = U.tokens_for(cfg, 70, 12)
+    eng = U.make_engine(path, device, page_size=16, pages=8)
+    want = _check(eng, cfg, W, toks, [[70], [50, 1]])
+    if device != "cpu":
+        e16 = U.make_engine(path, device, dtype="bfloat16", page_size=16, pages=8)
+        _check(e16, cfg, W, toks, [[33, 2, 1]], tol=U.TOL["bfloat16"], want=want)
+
+
 def test_bad_configs_are_refused(tmp_path):
     from dynamo_amd.models.registry import build_model, resolve_model_config
     later = U.make_config([U.latent_from(1), U.LATENT])
