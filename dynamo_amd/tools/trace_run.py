@@ -79,6 +79,7 @@ def main(argv=None) -> int:
     device = a.device
     if device == "auto":
         device = "cuda:0" if torch.cuda.is_available() else "cpu"
+    ensure_built(["_core"])      # the engine package itself imports it
     from dynamo_amd.models.registry import (native_extensions,
                                             resolve_model_config)
     model = resolve_model_config(a.model)
