@@ -393,7 +393,12 @@ def test_odd_sizes(tmp_path, device):
                          vocab=91, mult=1.0, eps=1e-3)
     toks = U.tokens_for(cfg, 40, 10)
     eng = U.make_engine(path, device, page_size=8, pages=12)
-    _check(eng, cfg, W, toks, [[40], [3, 1, 1, 19, 2]])
+    want = _check(eng, cfg, W, toks, [[40], [3, 1, 1, 19, 2]])
+    if device != "cpu":
+        e16 = U.make_engine(path, device, dtype="bfloat16", page_size=8,
+                            pages=12)
+        _check(e16, cfg, W, toks, [[40], [3, 1, 1, 19, 2]],
+               tol=U.TOL["bfloat16"], want=want)
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -662,6 +667,82 @@ def test_bf16_and_graph_decode(full_ckpt):
             assert e.graph_runner is not None and e.graph_runner.graphs
         outs.append(got)
     assert outs[0] == outs[1]
+
+
+MANY_HEADS = [
+    {"type": "latent_attention",
+     "mixer": {"heads": 8, "dim": 32, "rot_dim": 16, "vdim": 24, "kv_rank": 64,
+               "scale": 0.15, "rot": {"base": 5000.0, "dims": 16}},
+     "mlp": {"kind": "dense", "ff": 144}},
+    {"type": "attention",
+     "mixer": {"heads": 16, "kv_heads": 2, "dim": 16, "vdim": 24,
+               "scale": 0.25, "diff": 0.4, "mask": {"size": 37},
+               "rot": U.ROT_SCALED},
+     "mlp": None},
+    U.RGLRU,
+    {"type": "latent_attention",
+     "mixer": {"heads": 12, "dim": 16, "rot_dim": 16, "vdim": 8, "kv_rank": 64,
+               "scale": 0.2, "kv_from": 0,
+               "rot": {"base": 5000.0, "dims": 16}},
+     "mlp": {"kind": "dense", "ff": 120}},
+]
+
+
+@pytest.mark.gpu
+def test_bf16_many_heads_mixed_batches_and_graphs(tmp_path):
+    """Head groups of 8 and more in bf16: prompt tiles and decoded tokens
+    both run on the matrix cores, side by side in mixed batches over a
+    small pool, and in captured decode graphs."""
+    from dynamo_amd.engine import SamplingParams
+    path, cfg, W = _case(tmp_path, MANY_HEADS, seed=31, width=128)
+    lens = {"a": 150, "b": 9, "c": 77, "d": 1, "e": 66}
+    toks = {k: U.tokens_for(cfg, n, 70 + i) for i, (k, n) in enumerate(lens.items())}
+    want = {k: oracle.forward(cfg, W, t) for k, t in toks.items()}
+    eng = U.make_engine(path, "cuda:0", dtype="bfloat16", pages=22, slots=3,
+                        page_size=16)
+    plan = [[("a", 70), ("b", 5), ("d", 1)],
+            [("a", 1), ("b", 1)],
+            [("a", 1), ("b", 1), ("c", 64)],
+            [("a", 66), ("b", 2), ("c", 1)],
+            [("a", 1), ("c", 12), ("e", 65)],
+            [("a", 1), ("e", 1)],
+            [("a", 10)]]
+    at = {k: 0 for k in lens}
+    got = {k: [] for k in lens}
+    for step in plan:
+        entries, end = [], []
+        for rid, n in step:
+            entries.append((rid, toks[rid][at[rid]:at[rid] + n], list(range(n))))
+            at[rid] += n
+            if at[rid] == lens[rid]:
+                end.append(rid)
+        lg = eng.replay_step(entries, end).cpu()
+        row = 0
+        for rid, n in step:
+            got[rid].append(lg[row:row + n])
+            row += n
+    assert at == lens
+    for rid in lens:
+        assert U.rel_err(torch.cat(got[rid]), want[rid]) < U.TOL["bfloat16"], rid
+    # greedy decoding through captured graphs stays on the oracle's best
+    # tokens (up to bf16 noise in near ties)
+    e = U.make_engine(path, "cuda:0", dtype="bfloat16", graphs=True, slots=4,
+                      pages=40, page_size=16)
+    prompts = {f"g{i}": U.tokens_for(cfg, 30 + 17 * i, 90 + i) for i in range(3)}
+    for rid, p in prompts.items():
+        e.add_request(rid, p, SamplingParams(max_tokens=24, ignore_eos=True))
+    out = {k: [] for k in prompts}
+    while e.has_work():
+        for so in e.step():
+            out[so.req_id].append(so.new_token)
+    assert e.graph_runner is not None and e.graph_runner.graphs
+    for rid, p in prompts.items():
+        seq = list(p)
+        for tok in out[rid]:
+            lg = oracle.forward(cfg, W, seq)[-1]
+            spread = float(lg.std())
+            assert lg[tok] >= lg.max() - 0.15 * spread, (rid, len(seq))
+            seq.append(tok)
 
 
 # -- generation through the engine's own entry point ------------------------
