@@ -163,12 +163,21 @@ __global__ void xielu_kernel(T* __restrict__ out, const T* __restrict__ x,
   out[i] = from_f<T>(xielu_f(to_f(x[i]), ap, aq));
 }
 
-// Rotation of one pair at angle pos * freq. fp32 throughout.
-DEVINL void rot_pair(float a, float b, float ang, float& ra, float& rb) {
+// Rotation of one pair at angle pos * f, fp32 throughout. The frequency
+// comes as a float pair f = hi + lo; the rounding error of pos * hi is
+// recovered with an fma and, with pos * lo, applied as a first-order
+// correction to sin and cos, so the angle is good to about 1e-7 rad also
+// at positions in the tens of thousands (a plain fp32 product is off by
+// up to 6e-8 of the angle itself).
+DEVINL void rot_pair(float a, float b, float pos, float fhi, float flo,
+                     float& ra, float& rb) {
+  const float ang = pos * fhi;
+  const float rest = fmaf(pos, fhi, -ang) + pos * flo;
   float sn, cs;
   sincosf(ang, &sn, &cs);
-  ra = a * cs - b * sn;
-  rb = b * cs + a * sn;
+  const float s2 = fmaf(rest, cs, sn), c2 = fmaf(-rest, sn, cs);
+  ra = a * c2 - b * s2;
+  rb = b * c2 + a * s2;
 }
 
 // Partial rotary over `nvec` vectors of `len` entries per token row: the
@@ -191,8 +200,8 @@ __global__ void rope_rows_kernel(
     const int ia = interleaved ? 2 * i : i;
     const int ib = interleaved ? 2 * i + 1 : i + half;
     float ra, rb;
-    rot_pair(to_f(s[v * src_vec + ia]), to_f(s[v * src_vec + ib]),
-             pos * freqs[i], ra, rb);
+    rot_pair(to_f(s[v * src_vec + ia]), to_f(s[v * src_vec + ib]), pos,
+             freqs[i], freqs[half + i], ra, rb);
     d[v * dst_vec + ia] = from_f<T>(ra);
     d[v * dst_vec + ib] = from_f<T>(rb);
   }
@@ -232,8 +241,8 @@ __global__ void latent_append_kernel(
     const int ia = interleaved ? 2 * i : i;
     const int ib = interleaved ? 2 * i + 1 : i + half;
     float ra, rb;
-    rot_pair(to_f(src[rank + ia]), to_f(src[rank + ib]), pos * freqs[i], ra,
-             rb);
+    rot_pair(to_f(src[rank + ia]), to_f(src[rank + ib]), pos, freqs[i],
+             freqs[half + i], ra, rb);
     dst[rank + ia] = from_f<T>(ra);
     dst[rank + ib] = from_f<T>(rb);
   }
@@ -513,7 +522,8 @@ void rope_rows(torch::Tensor dst, int64_t dst_col, int64_t dst_vec,
                torch::Tensor positions, torch::Tensor freqs, int64_t nvec,
                int64_t len, bool interleaved) {
   const int T_ = src.size(0);
-  const int dims = 2 * freqs.numel();
+  SEQ_CHECK(freqs.dim() == 2 && freqs.size(0) == 2, "frequencies [2, dims/2]");
+  const int dims = 2 * freqs.size(1);
   SEQ_CHECK(src.dim() == 2 && dst.dim() == 2 && src.stride(1) == 1 &&
                 dst.stride(1) == 1 && dst.size(0) == T_ &&
                 dst.scalar_type() == src.scalar_type(), "rope rows");
@@ -548,7 +558,8 @@ void latent_append(torch::Tensor cache, torch::Tensor z, int64_t z_col,
   // cache [pages, 1, page_size, rank + rd]
   const int T_ = z.size(0);
   const int rank = norm_w.numel(), rd = cache.size(3) - rank;
-  const int dims = 2 * freqs.numel();
+  SEQ_CHECK(freqs.dim() == 2 && freqs.size(0) == 2, "frequencies [2, dims/2]");
+  const int dims = 2 * freqs.size(1);
   SEQ_CHECK(cache.dim() == 4 && cache.is_contiguous() && cache.size(1) == 1 &&
                 cache.scalar_type() == z.scalar_type() && rd >= 0,
             "latent cache");

@@ -325,12 +325,13 @@ class ClampedGLU(torch.nn.Module):
 
 
 def rotary_frequencies(rot: dict) -> torch.Tensor:
-    """fp32 [dims/2] angular frequencies base^(-2i/dims) of a rotary spec
-    {"base", "dims", "scaling"?}. The optional scaling {factor, low, high,
-    original} slows long wavelengths (above original/low) by `factor`,
-    keeps short ones (below original/high) and blends linearly in between.
-    Evaluated in float64, stored in fp32; angles are position * frequency
-    in fp32 inside the kernels."""
+    """fp32 [2, dims/2]: angular frequencies base^(-2i/dims) of a rotary
+    spec {"base", "dims", "scaling"?} as float pairs (row 0 + row 1). The
+    optional scaling {factor, low, high, original} slows long wavelengths
+    (above original/low) by `factor`, keeps short ones (below
+    original/high) and blends linearly in between. Evaluated in float64;
+    the kernels form position * frequency in fp32 with the pair's low part
+    and the product's rounding error as a correction."""
     import math
     n = int(rot["dims"])
     f = [float(rot["base"]) ** (-2.0 * i / n) for i in range(n // 2)]
@@ -345,7 +346,10 @@ def rotary_frequencies(rot: dict) -> torch.Tensor:
             elif wl >= lo_wl:
                 s = (sc["original"] / wl - sc["low"]) / (sc["high"] - sc["low"])
                 f[i] = (1 - s) * fi / sc["factor"] + s * fi
-    return torch.tensor(f, dtype=torch.float64).to(torch.float32)
+    f64 = torch.tensor(f, dtype=torch.float64)
+    hi = f64.to(torch.float32)
+    lo = (f64 - hi.double()).to(torch.float32)
+    return torch.stack([hi, lo])
 
 
 class RGLRUMixer(torch.nn.Module):
@@ -434,7 +438,7 @@ class DifferentialAttention(torch.nn.Module):
         # fused rows: q | k | v | gate
         self.w_in = init.mat(self.off_g + heads * vdim, width)
         self.freqs = rotary_frequencies(rot).to(init.device)
-        if 2 * self.freqs.numel() > dim:
+        if 2 * self.freqs.shape[1] > dim:
             raise ValueError("rotary dims exceed the head size")
         self.lq1, self.lk1 = init.vec(dim, -0.3, 0.3), init.vec(dim, -0.3, 0.3)
         self.lq2, self.lk2 = init.vec(dim, -0.3, 0.3), init.vec(dim, -0.3, 0.3)
@@ -493,7 +497,7 @@ class LatentAttention(torch.nn.Module):
         self.rank, self.scale, self.eps = rank, scale, eps
         self.shared_cache = shared_cache
         self.freqs = rotary_frequencies(rot).to(init.device)
-        if 2 * self.freqs.numel() > rot_dim:
+        if 2 * self.freqs.shape[1] > rot_dim:
             raise ValueError("rotary dims exceed the rotated part")
         self.off_z = heads * (dim + rot_dim)
         self.off_g = self.off_z + (0 if shared_cache else rank + rot_dim)

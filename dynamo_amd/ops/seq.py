@@ -265,8 +265,9 @@ def rope_rows(dst, dst_col: int, dst_vec: int, src, src_col: int,
               src_vec: int, positions, freqs, nvec: int, length: int,
               interleaved: bool):
     """For each token row, `nvec` vectors of `length` entries (vector v at
-    column col + v * vec) go from src to dst with their first
-    2 * len(freqs) entries rotated by position * freqs; dst may be src."""
+    column col + v * vec) go from src to dst with their first dims entries
+    rotated by position * f, f = freqs[0] + freqs[1] (fp32 [2, dims/2], see
+    models.mixers.rotary_frequencies); dst may be src."""
     if src.is_cuda:
         hip_seq().rope_rows(dst, dst_col, dst_vec, src, src_col, src_vec,
                             positions, freqs, nvec, length, bool(interleaved))

@@ -256,10 +256,13 @@ def xielu(x, pq):
 
 
 def _rotate(x, positions, freqs, interleaved):
-    """x fp32 [T, n, len]; the first 2 * len(freqs) entries are rotated."""
-    dims = 2 * freqs.numel()
-    ang = positions.float()[:, None] * freqs[None, :]
-    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    """x fp32 [T, n, len]; freqs [2, dims/2] (hi, lo float pairs); the
+    first dims entries are rotated."""
+    dims = 2 * freqs.shape[1]
+    ang = positions.double()[:, None] * (freqs[0].double()
+                                         + freqs[1].double())[None, :]
+    c = torch.cos(ang).float()[:, None, :]
+    s = torch.sin(ang).float()[:, None, :]
     y = x.clone()
     if interleaved:
         a, b = x[..., 0:dims:2], x[..., 1:dims:2]
